@@ -1,0 +1,118 @@
+/* C ABI of libfq_gfx950.so: the MI355X (gfx950) fused blockwise-FP8 quantisation
+ * kernels.  Each entry point replaces the Triton launch(es) made by one Python
+ * wrapper of the reference (path:line of the wrapper is cited at each
+ * declaration; paths are relative to the reference checkout).
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer on the current HIP device; the library
+ *    never allocates or frees device memory and never synchronises;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *    calls only enqueue work on it;
+ *  - bf16 inputs are row-major and contiguous, 16-byte aligned;
+ *  - fp8 outputs are raw bytes (OCP e4m3fn when fp8_kind == FQ_E4M3, OCP e5m2
+ *    when FQ_E5M2); scales are fp32 "scale_inv": value ~= code * scale,
+ *    scale = max(amax/fmax, 1e-30), rounded up to a power of two if round_scale;
+ *  - output_mode: 0 = row-wise (1x128) outputs only, 1 = transposed (128x1)
+ *    outputs only, 2 = both.  Outputs a mode does not produce may be NULL;
+ *  - return value: FQ_OK or a negative FQ_ERR_* code; fq_last_error() gives
+ *    the message of the calling thread's last failure.
+ *
+ * Layouts (nb = n/128, rb = r/128, b = c/128; element offsets):
+ *   single matrix: q[r*n + c], s[b*M + r], qt[c*M + r], st[rb*n + c]
+ *   per expert e (rows si..si+ce, tb = sum of ceil(c_e'/128) over e' < e):
+ *     q[(si+i)*n + c], s[si*nb + b*ce + i], qt[si*n + c*ce + i],
+ *     st[(tb + i/128)*n + c]
+ */
+#ifndef FQ_API_H_
+#define FQ_API_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FQ_OK 0
+#define FQ_ERR_ARG (-1)     /* null pointer, bad flag, misaligned pointer */
+#define FQ_ERR_SHAPE (-2)   /* shape outside what the kernels support */
+#define FQ_ERR_LAUNCH (-3)  /* HIP reported a launch failure */
+
+#define FQ_E4M3 0
+#define FQ_E5M2 1
+/* fq_group_quant only: e5m2 codes, scale = amax/448 (what the reference's group
+ * quantiser computes when its dtype argument is float8_e5m2,
+ * linghe/quant/group.py:27,57) */
+#define FQ_E5M2_MAX448 2
+
+/* library version (major*10000 + minor*100 + patch) */
+int fq_version(void);
+/* message of this thread's last failing call ("" if none) */
+const char* fq_last_error(void);
+
+/* triton_blockwise_quant, linghe/quant/block.py:129-170.
+ * x bf16 [M,N], N % 128 == 0.  q [M,N], s [N/128, M], qt [N, M], st [ceil(M/128), N]. */
+int fq_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t N,
+                       int round_scale, int output_mode, int fp8_kind, void* stream);
+
+/* triton_batch_blockwise_quant, linghe/quant/block.py:251-297.
+ * counts: device int32/int64 [n_experts]; total_blocks = sum ceil(count_e/128)
+ * computed by the caller from its host-side copy of the counts. */
+int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
+                               int64_t total_blocks, void* q, float* s, void* qt, float* st, int64_t M,
+                               int64_t N, int round_scale, int fp8_kind, void* stream);
+
+/* triton_group_quant, linghe/quant/group.py:40-63.  s is [M, N/128] row-major. */
+int fq_group_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
+                   void* stream);
+
+/* triton_rms_norm_forward, linghe/utils/norm.py:58-93.  out bf16 [M,n].
+ * reuse_rstd != 0: rstd [M] is an input, else it is written. */
+int fq_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* rstd, int64_t M, int64_t n, float eps,
+                   int reuse_rstd, void* stream);
+
+/* number of fp32 [n] partial rows fq_rmsnorm_bwd needs in dgamma_partials */
+int64_t fq_rmsnorm_bwd_num_partials(int64_t M, int64_t n);
+
+/* triton_rms_norm_backward, linghe/utils/norm.py:144-179.
+ * rstd may be NULL (recomputed).  dx bf16 [M,n], dgamma fp32 [n],
+ * dgamma_partials fp32 [n_partials, n] scratch (the reference's tmp_dw). */
+int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx, float* dgamma,
+                   float* dgamma_partials, int64_t n_partials, int64_t M, int64_t n, float eps, void* stream);
+
+/* triton_rms_norm_and_block_quant_forward, linghe/utils/norm.py:343-502.
+ * mode 0: writes q, s, rstd.  mode 1: reads rstd, writes qt, st.
+ * mode 2: writes q, s, rstd, qt, st. */
+int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt, float* st,
+                         int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
+                         void* stream);
+
+/* triton_silu_and_block_quant_forward, linghe/utils/silu.py:279-335.
+ * x bf16 [M, 2n] (gate | up).  Outputs as fq_blockwise_quant with N = n. */
+int fq_swiglu_quant_fwd(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t n,
+                        int round_scale, int output_mode, int fp8_kind, void* stream);
+
+/* triton_silu_and_block_quant_backward, linghe/utils/silu.py:424-464.
+ * g bf16 [M,n], x bf16 [M,2n].  dq [M,2n] (dx1|dx2), ds [2n/128, M],
+ * dqt [2n, M], dst [ceil(M/128), 2n]. */
+int fq_swiglu_quant_bwd(const void* g, const void* x, void* dq, float* ds, void* dqt, float* dst, int64_t M,
+                        int64_t n, int round_scale, int fp8_kind, void* stream);
+
+/* triton_batch_weighted_silu_and_block_quant_forward, linghe/utils/silu.py:797-950.
+ * weight [M] fp32 (or bf16 when weight_is_bf16), per-expert packed outputs. */
+int fq_batched_swiglu_quant_fwd(const void* x, const void* weight, int weight_is_bf16, const void* counts,
+                                int counts_is_i64, int n_experts, int64_t total_blocks, void* q, float* s,
+                                void* qt, float* st, int64_t M, int64_t n, int round_scale, int output_mode,
+                                int fp8_kind, void* stream);
+
+/* triton_batch_weighted_silu_and_block_quant_backward, linghe/utils/silu.py:1293-1393.
+ * dw [M] in the weight's dtype; dw_partials fp32 [M, n/128] scratch (the
+ * reference's dws). */
+int fq_batched_swiglu_quant_bwd(const void* g, const void* x, const void* weight, int weight_is_bf16,
+                                const void* counts, int counts_is_i64, int n_experts, int64_t total_blocks,
+                                void* dq, float* ds, void* dw, void* dqt, float* dst, float* dw_partials,
+                                int64_t M, int64_t n, int round_scale, int fp8_kind, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FQ_API_H_ */

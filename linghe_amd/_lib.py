@@ -1,0 +1,91 @@
+"""ctypes binding of libfq_gfx950.so (declared in include/fq_api.h).
+
+The library is the only compute path: if it is missing or fails to load, the
+import of any operator module raises; there is no eager / CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libfq_gfx950.so"
+LIB_PATH = os.path.join(_HERE, LIB_NAME)
+
+FQ_E4M3 = 0
+FQ_E5M2 = 1
+FQ_E5M2_MAX448 = 2
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_L = ctypes.c_int64
+_F = ctypes.c_float
+
+# name -> argtypes, exactly the declarations of include/fq_api.h
+SIGNATURES = {
+    "fq_blockwise_quant": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
+    "fq_batched_blockwise_quant": [_P, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _P],
+    "fq_group_quant": [_P, _P, _P, _L, _L, _I, _I, _P],
+    "fq_rmsnorm_fwd": [_P, _P, _P, _P, _L, _L, _F, _I, _P],
+    "fq_rmsnorm_bwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _P],
+    "fq_rmsnorm_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _I, _I, _P],
+    "fq_swiglu_quant_fwd": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
+    "fq_swiglu_quant_bwd": [_P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
+    "fq_batched_swiglu_quant_fwd": [_P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
+    "fq_batched_swiglu_quant_bwd": [_P, _P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
+}
+OTHER_SYMBOLS = ["fq_version", "fq_last_error", "fq_rmsnorm_bwd_num_partials"]
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m linghe_amd.build` "
+            "(hipcc, gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = _I
+    lib.fq_version.argtypes = []
+    lib.fq_version.restype = _I
+    lib.fq_last_error.argtypes = []
+    lib.fq_last_error.restype = ctypes.c_char_p
+    lib.fq_rmsnorm_bwd_num_partials.argtypes = [_L, _L]
+    lib.fq_rmsnorm_bwd_num_partials.restype = _L
+    return lib
+
+
+lib = _load()
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = lib.fq_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"libfq_gfx950 error {rc}: {msg}")
+
+
+def ptr(t):
+    """Device address of a tensor (None -> NULL)."""
+    return None if t is None else t.data_ptr()
+
+
+def stream_of(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def fp8_kind(dtype) -> int:
+    if dtype == torch.float8_e4m3fn:
+        return FQ_E4M3
+    if dtype == torch.float8_e5m2:
+        return FQ_E5M2
+    raise ValueError(f"unsupported fp8 dtype {dtype}")
+
+
+def require_device_bf16(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU: the HIP kernels are the only implementation")
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16, got {t.dtype}")

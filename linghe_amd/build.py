@@ -1,0 +1,74 @@
+"""Build libfq_gfx950.so (the C-ABI library with the gfx950 kernels) in-tree.
+
+    python -m linghe_amd.build
+
+hipcc cross-compiles for gfx950 without a GPU.  The three translation units are
+compiled in parallel and linked into ``linghe_amd/libfq_gfx950.so``.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_NAME = "libfq_gfx950.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+SOURCES = ["fq_api.hip", "fq_tile_kernels.hip", "fq_row_kernels.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    # parity with the fp32 CPU oracle needs separate mul/add roundings
+    "-ffp-contract=off",
+    # packed fp32 VALU ops are not to be generated for this machine pool
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    # the host pass does not know the -packed-fp32-ops feature and says so: harmless
+    err = "\n".join(l for l in proc.stderr.splitlines() if "not a recognized feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), proc.stdout, err))
+    if err.strip():
+        sys.stderr.write(err + "\n")
+
+
+def build_library(extra_flags=(), verbose: bool = False) -> str:
+    hipcc = _hipcc()
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd))
+        _run(cmd)
+
+    with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
+        list(pool.map(compile_one, zip(SOURCES, objs)))
+    tmp = LIB_PATH + ".tmp"
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

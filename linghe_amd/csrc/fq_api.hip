@@ -1,0 +1,246 @@
+// C-ABI layer: argument validation + dispatch to the kernel launchers.
+// Holds no mutable global state besides the per-thread error message.
+#include "../../include/fq_api.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "fq_launch.h"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(hipError_t e, const char* what) {
+  if (e == hipSuccess) return FQ_OK;
+  return fail(FQ_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+#define FQ_REQUIRE(cond, code, ...) \
+  do { if (!(cond)) return fail(code, __VA_ARGS__); } while (0)
+
+int check_common(const char* fn, int64_t M, int64_t width, int round_scale, int fp8_kind) {
+  FQ_REQUIRE(M >= 0, FQ_ERR_SHAPE, "%s: negative row count", fn);
+  FQ_REQUIRE(width > 0 && width % 128 == 0, FQ_ERR_SHAPE, "%s: width %lld is not a positive multiple of 128", fn,
+             (long long)width);
+  FQ_REQUIRE(width <= (1 << 24), FQ_ERR_SHAPE, "%s: width too large", fn);
+  FQ_REQUIRE(M <= ((int64_t)1 << 31) - 256, FQ_ERR_SHAPE, "%s: too many rows", fn);
+  FQ_REQUIRE(round_scale == 0 || round_scale == 1, FQ_ERR_ARG, "%s: round_scale must be 0 or 1", fn);
+  FQ_REQUIRE(fp8_kind == FQ_E4M3 || fp8_kind == FQ_E5M2, FQ_ERR_ARG, "%s: unknown fp8_kind %d", fn, fp8_kind);
+  return FQ_OK;
+}
+
+int check_mode_ptrs(const char* fn, int mode, const void* q, const void* s, const void* qt, const void* st) {
+  FQ_REQUIRE(mode >= 0 && mode <= 2, FQ_ERR_ARG, "%s: output_mode must be 0, 1 or 2", fn);
+  if (mode != 1) FQ_REQUIRE(q && s, FQ_ERR_ARG, "%s: row-wise outputs are NULL", fn);
+  if (mode != 0) FQ_REQUIRE(qt && st, FQ_ERR_ARG, "%s: transposed outputs are NULL", fn);
+  if (q) FQ_REQUIRE((reinterpret_cast<uintptr_t>(q) & 7u) == 0, FQ_ERR_ARG, "%s: q must be 8-byte aligned", fn);
+  return FQ_OK;
+}
+
+int check_tiles(const char* fn, int64_t tiles) {
+  FQ_REQUIRE(tiles < ((int64_t)1 << 31), FQ_ERR_SHAPE, "%s: too many tiles for one launch", fn);
+  return FQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fq_version(void) { return 100; }
+
+const char* fq_last_error(void) { return g_err; }
+
+int fq_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t N,
+                       int round_scale, int output_mode, int fp8_kind, void* stream) {
+  const char* fn = "fq_blockwise_quant";
+  int rc = check_common(fn, M, N, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, output_mode, q, s, qt, st))) return rc;
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && aligned16(x), FQ_ERR_ARG, "%s: x is NULL or not 16-byte aligned", fn);
+  const int64_t rbs = (M + 127) / 128;
+  if ((rc = check_tiles(fn, rbs * (N / 128)))) return rc;
+  return check_launch(fq::launch_blockwise_quant(x, q, s, qt, st, M, (int)N, round_scale, output_mode, fp8_kind,
+                                                 nullptr, 0, 0, rbs, (hipStream_t)stream),
+                      fn);
+}
+
+int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
+                               int64_t total_blocks, void* q, float* s, void* qt, float* st, int64_t M,
+                               int64_t N, int round_scale, int fp8_kind, void* stream) {
+  const char* fn = "fq_batched_blockwise_quant";
+  int rc = check_common(fn, M, N, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, 2, q, s, qt, st))) return rc;
+  FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0, FQ_ERR_SHAPE, "%s: negative expert/block count", fn);
+  if (M == 0 || total_blocks == 0) return FQ_OK;
+  FQ_REQUIRE(x && aligned16(x) && counts, FQ_ERR_ARG, "%s: x/counts NULL or x misaligned", fn);
+  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
+  if ((rc = check_tiles(fn, total_blocks * (N / 128)))) return rc;
+  return check_launch(fq::launch_blockwise_quant(x, q, s, qt, st, M, (int)N, round_scale, 2, fp8_kind, counts,
+                                                 counts_is_i64 != 0, n_experts, total_blocks, (hipStream_t)stream),
+                      fn);
+}
+
+int fq_group_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
+                   void* stream) {
+  const char* fn = "fq_group_quant";
+  int rc = check_common(fn, M, N, round_scale, fp8_kind == FQ_E5M2_MAX448 ? FQ_E5M2 : fp8_kind);
+  if (rc) return rc;
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && aligned16(x) && q && s, FQ_ERR_ARG, "%s: NULL or misaligned pointer", fn);
+  FQ_REQUIRE((reinterpret_cast<uintptr_t>(q) & 7u) == 0, FQ_ERR_ARG, "%s: q must be 8-byte aligned", fn);
+  return check_launch(fq::launch_group_quant(x, q, s, M * (N / 128), round_scale, fp8_kind, (hipStream_t)stream), fn);
+}
+
+static int check_norm_shape(const char* fn, int64_t M, int64_t n) {
+  FQ_REQUIRE(M >= 0, FQ_ERR_SHAPE, "%s: negative row count", fn);
+  FQ_REQUIRE(n > 0 && n % 8 == 0 && n <= 8192, FQ_ERR_SHAPE,
+             "%s: hidden size %lld must be a multiple of 8 and at most 8192", fn, (long long)n);
+  FQ_REQUIRE(M <= ((int64_t)1 << 31) - 256, FQ_ERR_SHAPE, "%s: too many rows", fn);
+  return FQ_OK;
+}
+
+int fq_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* rstd, int64_t M, int64_t n, float eps,
+                   int reuse_rstd, void* stream) {
+  const char* fn = "fq_rmsnorm_fwd";
+  int rc = check_norm_shape(fn, M, n);
+  if (rc) return rc;
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && gamma && out && rstd, FQ_ERR_ARG, "%s: NULL pointer", fn);
+  FQ_REQUIRE(aligned16(x) && aligned16(gamma) && aligned16(out), FQ_ERR_ARG, "%s: misaligned pointer", fn);
+  return check_launch(fq::launch_rmsnorm_fwd(x, gamma, out, nullptr, rstd, M, (int)n, eps, reuse_rstd != 0, 0, 0,
+                                             FQ_E4M3, (hipStream_t)stream),
+                      fn);
+}
+
+int64_t fq_rmsnorm_bwd_num_partials(int64_t M, int64_t n) {
+  (void)n;
+  return fq::rmsnorm_bwd_partials(M);
+}
+
+int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx, float* dgamma,
+                   float* dgamma_partials, int64_t n_partials, int64_t M, int64_t n, float eps, void* stream) {
+  const char* fn = "fq_rmsnorm_bwd";
+  int rc = check_norm_shape(fn, M, n);
+  if (rc) return rc;
+  FQ_REQUIRE(dgamma && dgamma_partials, FQ_ERR_ARG, "%s: dgamma outputs are NULL", fn);
+  FQ_REQUIRE(n_partials == fq::rmsnorm_bwd_partials(M), FQ_ERR_SHAPE,
+             "%s: n_partials must equal fq_rmsnorm_bwd_num_partials(M, n)", fn);
+  if (M > 0) {
+    FQ_REQUIRE(dy && x && gamma && dx, FQ_ERR_ARG, "%s: NULL pointer", fn);
+    FQ_REQUIRE(aligned16(dy) && aligned16(x) && aligned16(gamma) && aligned16(dx) && aligned16(dgamma_partials),
+               FQ_ERR_ARG, "%s: misaligned pointer", fn);
+  }
+  return check_launch(fq::launch_rmsnorm_bwd(dy, x, gamma, rstd, dx, dgamma, dgamma_partials, n_partials, M, (int)n,
+                                             eps, (hipStream_t)stream),
+                      fn);
+}
+
+int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt, float* st,
+                         int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
+                         void* stream) {
+  const char* fn = "fq_rmsnorm_quant_fwd";
+  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_norm_shape(fn, M, n))) return rc;
+  if ((rc = check_mode_ptrs(fn, output_mode, q, s, qt, st))) return rc;
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && gamma && rstd, FQ_ERR_ARG, "%s: NULL pointer", fn);
+  FQ_REQUIRE(aligned16(x) && aligned16(gamma), FQ_ERR_ARG, "%s: misaligned pointer", fn);
+  hipStream_t st_ = (hipStream_t)stream;
+  if (output_mode == 0 || output_mode == 2) {
+    rc = check_launch(fq::launch_rmsnorm_fwd(x, gamma, q, s, rstd, M, (int)n, eps, 0, 1, round_scale, fp8_kind, st_),
+                      fn);
+    if (rc) return rc;
+  }
+  if (output_mode == 1 || output_mode == 2) {
+    if ((rc = check_tiles(fn, ((M + 127) / 128) * (n / 128)))) return rc;
+    rc = check_launch(fq::launch_rmsnorm_quant_tile(x, gamma, rstd, nullptr, nullptr, qt, st, M, (int)n, round_scale,
+                                                    1, fp8_kind, st_),
+                      fn);
+  }
+  return rc;
+}
+
+int fq_swiglu_quant_fwd(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t n,
+                        int round_scale, int output_mode, int fp8_kind, void* stream) {
+  const char* fn = "fq_swiglu_quant_fwd";
+  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, output_mode, q, s, qt, st))) return rc;
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && aligned16(x), FQ_ERR_ARG, "%s: x is NULL or not 16-byte aligned", fn);
+  const int64_t rbs = (M + 127) / 128;
+  if ((rc = check_tiles(fn, rbs * (n / 128)))) return rc;
+  return check_launch(fq::launch_silu_quant_fwd(x, nullptr, 0, q, s, qt, st, M, (int)n, round_scale, output_mode,
+                                                fp8_kind, nullptr, 0, 0, rbs, (hipStream_t)stream),
+                      fn);
+}
+
+int fq_swiglu_quant_bwd(const void* g, const void* x, void* dq, float* ds, void* dqt, float* dst, int64_t M,
+                        int64_t n, int round_scale, int fp8_kind, void* stream) {
+  const char* fn = "fq_swiglu_quant_bwd";
+  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, 2, dq, ds, dqt, dst))) return rc;
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(g && x && aligned16(g) && aligned16(x), FQ_ERR_ARG, "%s: NULL or misaligned input", fn);
+  const int64_t rbs = (M + 127) / 128;
+  if ((rc = check_tiles(fn, rbs * (n / 128)))) return rc;
+  return check_launch(fq::launch_silu_quant_bwd(g, x, nullptr, 0, dq, ds, dqt, dst, nullptr, nullptr, M, (int)n,
+                                                round_scale, fp8_kind, nullptr, 0, 0, rbs, (hipStream_t)stream),
+                      fn);
+}
+
+int fq_batched_swiglu_quant_fwd(const void* x, const void* weight, int weight_is_bf16, const void* counts,
+                                int counts_is_i64, int n_experts, int64_t total_blocks, void* q, float* s,
+                                void* qt, float* st, int64_t M, int64_t n, int round_scale, int output_mode,
+                                int fp8_kind, void* stream) {
+  const char* fn = "fq_batched_swiglu_quant_fwd";
+  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, output_mode, q, s, qt, st))) return rc;
+  FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0, FQ_ERR_SHAPE, "%s: negative expert/block count", fn);
+  if (M == 0 || total_blocks == 0) return FQ_OK;
+  FQ_REQUIRE(x && aligned16(x) && weight && counts, FQ_ERR_ARG, "%s: NULL or misaligned input", fn);
+  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
+  if ((rc = check_tiles(fn, total_blocks * (n / 128)))) return rc;
+  return check_launch(fq::launch_silu_quant_fwd(x, weight, weight_is_bf16 != 0, q, s, qt, st, M, (int)n, round_scale,
+                                                output_mode, fp8_kind, counts, counts_is_i64 != 0, n_experts,
+                                                total_blocks, (hipStream_t)stream),
+                      fn);
+}
+
+int fq_batched_swiglu_quant_bwd(const void* g, const void* x, const void* weight, int weight_is_bf16,
+                                const void* counts, int counts_is_i64, int n_experts, int64_t total_blocks,
+                                void* dq, float* ds, void* dw, void* dqt, float* dst, float* dw_partials,
+                                int64_t M, int64_t n, int round_scale, int fp8_kind, void* stream) {
+  const char* fn = "fq_batched_swiglu_quant_bwd";
+  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, 2, dq, ds, dqt, dst))) return rc;
+  FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0, FQ_ERR_SHAPE, "%s: negative expert/block count", fn);
+  if (M == 0 || total_blocks == 0) return FQ_OK;
+  FQ_REQUIRE(g && x && aligned16(g) && aligned16(x) && weight && counts && dw && dw_partials, FQ_ERR_ARG,
+             "%s: NULL or misaligned pointer", fn);
+  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
+  if ((rc = check_tiles(fn, total_blocks * (n / 128)))) return rc;
+  return check_launch(fq::launch_silu_quant_bwd(g, x, weight, weight_is_bf16 != 0, dq, ds, dqt, dst, dw_partials, dw,
+                                                M, (int)n, round_scale, fp8_kind, counts, counts_is_i64 != 0,
+                                                n_experts, total_blocks, (hipStream_t)stream),
+                      fn);
+}
+
+}  // extern "C"

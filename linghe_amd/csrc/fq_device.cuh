@@ -1,0 +1,172 @@
+// Device-side building blocks for the fused blockwise-FP8 quantisation kernels
+// (gfx950 / CDNA4, wave64).  No MFMA: every kernel on this path is HBM-bound.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fq {
+
+constexpr int kGroup = 128;           // 1x128 / 128x1 quantisation group
+constexpr float kScaleFloor = 1e-30f;  // linghe/tools/util.py:58-60
+
+// FP8 flavours. E4M3 = OCP e4m3fn (max 448), E5M2 = OCP e5m2 (max 57344).
+// kE5M2Max448 = e5m2 codes with the scale still derived from 448, which is what
+// the reference's group quantiser does when asked for e5m2
+// (linghe/quant/group.py:27 divides by 448.0 whatever the output dtype).
+enum Fp8Kind : int { kE4M3 = 0, kE5M2 = 1, kE5M2Max448 = 2 };
+template <int KIND> struct Fp8Traits;
+template <> struct Fp8Traits<kE4M3> { static constexpr float kMax = 448.0f; static constexpr bool kBf8 = false; };
+template <> struct Fp8Traits<kE5M2> { static constexpr float kMax = 57344.0f; static constexpr bool kBf8 = true; };
+template <> struct Fp8Traits<kE5M2Max448> { static constexpr float kMax = 448.0f; static constexpr bool kBf8 = true; };
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// two bf16 packed in a dword -> fp32 (exact)
+__device__ __forceinline__ float bf16_lo(uint32_t p) { return as_f32(p << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t p) { return as_f32(p & 0xffff0000u); }
+
+// 8 packed bf16 (one 128-bit load) -> 8 fp32
+__device__ __forceinline__ void unpack8(const uint4& p, float (&v)[8]) {
+  v[0] = bf16_lo(p.x); v[1] = bf16_hi(p.x);
+  v[2] = bf16_lo(p.y); v[3] = bf16_hi(p.y);
+  v[4] = bf16_lo(p.z); v[5] = bf16_hi(p.z);
+  v[6] = bf16_lo(p.w); v[7] = bf16_hi(p.w);
+}
+
+// fp32 pair -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  floatx2_t f = {a, b};
+  bf16x2_t h = __builtin_convertvector(f, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, h);
+}
+__device__ __forceinline__ uint4 pack8_bf16(const float (&v)[8]) {
+  uint4 o;
+  o.x = pack_bf16x2(v[0], v[1]);
+  o.y = pack_bf16x2(v[2], v[3]);
+  o.z = pack_bf16x2(v[4], v[5]);
+  o.w = pack_bf16x2(v[6], v[7]);
+  return o;
+}
+
+// 4 fp32 -> 4 fp8 codes in one dword (native converts, RNE)
+template <int KIND>
+__device__ __forceinline__ uint32_t pack4_fp8(float a, float b, float c, float d) {
+  uint32_t w = 0;
+  if constexpr (!Fp8Traits<KIND>::kBf8) {
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  } else {
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, w, true);
+  }
+  return w;
+}
+
+// ---------------------------------------------------------------------------
+// exact division by a scale that is shared by many elements.
+// rcp:  one Newton step on v_rcp_f32 (correctly rounded but for ~1e-6 of inputs)
+// div:  q0 = v*r ; q = fma(fma(-q0, s, v), r, q0)  -> the correctly rounded v/s
+// (Markstein's correction; checked against IEEE division in the parity tests).
+// ---------------------------------------------------------------------------
+struct Divisor {
+  float s;  // the scale
+  float r;  // ~ 1/s
+};
+__device__ __forceinline__ Divisor make_divisor(float s) {
+  float r0 = __builtin_amdgcn_rcpf(s);
+  float e = __builtin_fmaf(-s, r0, 1.0f);
+  Divisor d;
+  d.s = s;
+  d.r = __builtin_fmaf(e, r0, r0);
+  return d;
+}
+__device__ __forceinline__ float div_exact(float v, const Divisor& d) {
+  float q0 = v * d.r;
+  float e = __builtin_fmaf(-q0, d.s, v);
+  return __builtin_fmaf(e, d.r, q0);
+}
+
+// exp2(ceil(log2(s))) as torch evaluates it in fp32 (linghe/tools/util.py:61-62):
+// the fp32 log2 of a value a few ulps above 2^e rounds to e itself, so such
+// values are NOT rounded up.  Reproduced with integer arithmetic: round up iff
+// log2(mantissa) exceeds half an fp32 ulp of the number line just above e.
+__device__ __forceinline__ float pow2_ceil_like_torch(float s) {
+  uint32_t b = as_u32(s);
+  int e = (int)((b >> 23) & 0xffu) - 127;
+  uint32_t k = b & 0x7fffffu;
+  if (k != 0) {
+    bool up = true;
+    if (e != 0) {
+      uint32_t ae = (uint32_t)(e < 0 ? -e : e);
+      int fl = 31 - __builtin_clz(ae);
+      bool pow2 = (ae & (ae - 1u)) == 0u;
+      int ulp_exp = fl - 23 - ((e < 0 && pow2) ? 1 : 0);
+      float half_ulp = as_f32((uint32_t)(ulp_exp - 1 + 127) << 23);
+      float delta = (float)k * (1.4426950408889634f * 0x1p-23f);
+      up = delta > half_ulp;
+    }
+    if (up) e += 1;
+  }
+  return as_f32((uint32_t)(e + 127) << 23);
+}
+
+// scale = max(amax / fmax, 1e-30) [rounded up to a power of two]
+template <int KIND, bool ROUND>
+__device__ __forceinline__ float make_scale(float amax) {
+  float s = fmaxf(amax / Fp8Traits<KIND>::kMax, kScaleFloor);
+  if constexpr (ROUND) s = pow2_ceil_like_torch(s);
+  return s;
+}
+
+// ---------------------------------------------------------------------------
+// DPP reductions inside a row of 16 lanes (a wave64 is four such rows).
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+  return as_f32((uint32_t)__builtin_amdgcn_update_dpp(0, (int)as_u32(v), CTRL, 0xf, 0xf, false));
+}
+constexpr int kDppQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+
+// every lane of the 16-lane row ends with the max over the row
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_mov<kDppQuadXor1>(v));
+  v = fmaxf(v, dpp_mov<kDppQuadXor2>(v));
+  v = fmaxf(v, dpp_mov<kDppRowHalfMirror>(v));
+  v = fmaxf(v, dpp_mov<kDppRowMirror>(v));
+  return v;
+}
+// every lane of the 16-lane row ends with the same sum (fixed order -> deterministic)
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_mov<kDppQuadXor1>(v);
+  v += dpp_mov<kDppQuadXor2>(v);
+  v += dpp_mov<kDppRowHalfMirror>(v);
+  v += dpp_mov<kDppRowMirror>(v);
+  return v;
+}
+// whole-wave sum / max, result in every lane
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = row16_max(v);
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  v = fmaxf(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+__device__ __forceinline__ float sigmoid_f32(float x) {
+  // 1 / (1 + exp(-x)) with a full-precision exp and a true division,
+  // the formula torch's CPU sigmoid evaluates
+  return 1.0f / (1.0f + expf(-x));
+}
+
+}  // namespace fq

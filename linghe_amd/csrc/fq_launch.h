@@ -1,0 +1,41 @@
+// Internal launcher prototypes shared between the kernel translation units and
+// the C-ABI layer.  Everything here takes raw device pointers and a stream and
+// only enqueues work.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fq {
+
+hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int N,
+                                  int round_scale, int mode, int kind, const void* counts, int counts_i64,
+                                  int n_experts, int64_t row_blocks, hipStream_t stream);
+
+hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_bf16, void* q, float* s, void* qt,
+                                 float* st, int64_t M, int n, int round_scale, int mode, int kind,
+                                 const void* counts, int counts_i64, int n_experts, int64_t row_blocks,
+                                 hipStream_t stream);
+
+hipError_t launch_silu_quant_bwd(const void* g, const void* x, const void* weight, int weight_bf16, void* q,
+                                 float* s, void* qt, float* st, float* dw_part, void* dw, int64_t M, int n,
+                                 int round_scale, int kind, const void* counts, int counts_i64, int n_experts,
+                                 int64_t row_blocks, hipStream_t stream);
+
+hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const float* rstd, void* q, float* s,
+                                     void* qt, float* st, int64_t M, int n, int round_scale, int mode, int kind,
+                                     hipStream_t stream);
+
+hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* scale, float* rstd, int64_t M,
+                              int n, float eps, int reuse_rstd, int quant, int round_scale, int kind,
+                              hipStream_t stream);
+
+int64_t rmsnorm_bwd_partials(int64_t M);
+
+hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
+                              float* dgamma, float* dg_part, int64_t n_partials, int64_t M, int n, float eps,
+                              hipStream_t stream);
+
+hipError_t launch_group_quant(const void* x, void* q, float* s, int64_t n_groups, int round_scale, int kind,
+                              hipStream_t stream);
+
+}  // namespace fq

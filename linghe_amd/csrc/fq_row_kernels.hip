@@ -1,0 +1,376 @@
+// Row kernels: a workgroup owns whole rows (the RMSNorm statistic needs the full
+// row) and keeps the row in registers between the reduction and the outputs, so
+// every element is read from HBM once.
+//   rmsnorm_fwd          bf16 RMSNorm                       (linghe/utils/norm.py:13-93)
+//   rmsnorm_quant_row    RMSNorm + row-wise 1x128 quant      (linghe/utils/norm.py:252-297)
+//   rmsnorm_bwd          dx (bf16) + dgamma partial sums      (linghe/utils/norm.py:96-179)
+//   colsum               dgamma = sum of the partials
+//   group_quant          row-wise 1x128 quant, scale [M, N/128] (linghe/quant/group.py:11-63)
+//
+// Thread t of a T-thread workgroup owns the 8-column chunks t, t+T, t+2T, ...
+// (one 128-bit load each); 16 consecutive lanes therefore share a 128-column
+// quantisation group.  The next row is prefetched while the current one is
+// processed.
+#include "fq_device.cuh"
+#include "fq_launch.h"
+
+namespace fq {
+
+template <int T>
+struct RowShared {
+  float red[2][2][T / 64];  // [parity][value][wave]
+};
+
+// sum of (a, b) over the workgroup, fixed order; one barrier per call
+template <int T>
+__device__ __forceinline__ void block_sum2(float& a, float& b, RowShared<T>& sh, int parity) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if constexpr (T > 64) {
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+      sh.red[parity][0][wave] = a;
+      sh.red[parity][1][wave] = b;
+    }
+    __syncthreads();
+    a = sh.red[parity][0][0];
+    b = sh.red[parity][1][0];
+#pragma unroll
+    for (int w = 1; w < T / 64; ++w) {
+      a += sh.red[parity][0][w];
+      b += sh.red[parity][1][w];
+    }
+  }
+}
+
+template <int T, int NCHUNK>
+__device__ __forceinline__ void load_row(const uint16_t* row, int n, uint4 (&raw)[NCHUNK]) {
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) {
+    const int c = threadIdx.x + k * T;
+    raw[k] = make_uint4(0, 0, 0, 0);
+    if (c * 8 < n) raw[k] = *(const uint4*)(row + c * 8);
+  }
+}
+
+__device__ __forceinline__ float rstd_from_sumsq(float ss, int n, float eps) {
+  // rsqrt(sum/n + eps) as the fp32 CPU oracle evaluates it: true division,
+  // correctly rounded sqrt, true reciprocal
+  return 1.0f / sqrtf(ss / (float)n + eps);
+}
+
+template <int NCHUNK>
+__device__ __forceinline__ float sumsq(const uint4 (&raw)[NCHUNK]) {
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) {
+    float a[8];
+    unpack8(raw[k], a);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(a[j], a[j], ss);
+  }
+  return ss;
+}
+
+// ---------------------------------------------------------------------------
+// forward: OUT_QUANT=false -> bf16 y ; OUT_QUANT=true -> fp8 codes + [nb, M] scales
+// ---------------------------------------------------------------------------
+template <int T, int NCHUNK, bool REUSE, bool OUT_QUANT, int KIND, bool ROUND>
+__global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restrict__ x,
+                                                        const uint16_t* __restrict__ gamma, void* __restrict__ out,
+                                                        float* __restrict__ scale, float* __restrict__ rstd,
+                                                        int64_t M, int n, float eps, int rows_per_wg) {
+  __shared__ RowShared<T> sh;
+  const int tid = threadIdx.x;
+  uint4 gm[NCHUNK];
+  load_row<T, NCHUNK>(gamma, n, gm);
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
+  int64_t r1 = r0 + rows_per_wg;
+  if (r1 > M) r1 = M;
+  if (r0 >= r1) return;
+
+  auto process = [&](const uint4 (&raw)[NCHUNK], int64_t row, int parity) {
+    float r;
+    if constexpr (REUSE) {
+      r = rstd[row];
+    } else {
+      float ss = sumsq<NCHUNK>(raw), dummy = 0.f;
+      block_sum2<T>(ss, dummy, sh, parity);
+      r = rstd_from_sumsq(ss, n, eps);
+      if (tid == 0) rstd[row] = r;
+    }
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      const int c = tid + k * T;
+      float a[8], w[8], y[8];
+      unpack8(raw[k], a);
+      unpack8(gm[k], w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = (a[j] * r) * w[j];
+      if constexpr (!OUT_QUANT) {
+        if (c * 8 < n) *(uint4*)((uint16_t*)out + row * n + c * 8) = pack8_bf16(y);
+      } else {
+        float m = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(y[j]));
+        m = row16_max(m);
+        const float sc = make_scale<KIND, ROUND>(m);
+        const Divisor d = make_divisor(sc);
+        float qv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qv[j] = div_exact(y[j], d);
+        uint2 pk;
+        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+        if (c * 8 < n) {
+          *(uint2*)((uint8_t*)out + row * n + c * 8) = pk;
+          if ((c & 15) == 0) scale[(int64_t)(c >> 4) * M + row] = sc;
+        }
+      }
+    }
+  };
+
+  uint4 bufA[NCHUNK], bufB[NCHUNK];
+  load_row<T, NCHUNK>(x + r0 * n, n, bufA);
+  for (int64_t row = r0; row < r1; row += 2) {
+    if (row + 1 < r1) load_row<T, NCHUNK>(x + (row + 1) * n, n, bufB);
+    process(bufA, row, 0);
+    if (row + 1 < r1) {
+      if (row + 2 < r1) load_row<T, NCHUNK>(x + (row + 2) * n, n, bufA);
+      process(bufB, row + 1, 1);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// backward: dx = r*g*w - r^3 * x * sum(x*g*w)/n ; dgamma partial += x*g*r
+// ---------------------------------------------------------------------------
+template <int T, int NCHUNK, bool REUSE>
+__global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ dy,
+                                                        const uint16_t* __restrict__ x,
+                                                        const uint16_t* __restrict__ gamma,
+                                                        const float* __restrict__ rstd_in,
+                                                        uint16_t* __restrict__ dx, float* __restrict__ dg_part,
+                                                        int64_t M, int n, float eps, int rows_per_wg) {
+  __shared__ RowShared<T> sh;
+  const int tid = threadIdx.x;
+  uint4 gm[NCHUNK];
+  load_row<T, NCHUNK>(gamma, n, gm);
+  float acc[NCHUNK][8];
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[k][j] = 0.f;
+
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
+  int64_t r1 = r0 + rows_per_wg;
+  if (r1 > M) r1 = M;
+
+  auto process = [&](const uint4 (&rx)[NCHUNK], const uint4 (&rg)[NCHUNK], int64_t row, int parity) {
+    float ss = 0.f, dot = 0.f;
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      float a[8], g[8], w[8];
+      unpack8(rx[k], a);
+      unpack8(rg[k], g);
+      unpack8(gm[k], w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        ss = __builtin_fmaf(a[j], a[j], ss);
+        dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
+      }
+    }
+    block_sum2<T>(ss, dot, sh, parity);
+    float r;
+    if constexpr (REUSE) r = rstd_in[row];
+    else r = rstd_from_sumsq(ss, n, eps);
+    const float coef = ((r * r) * r) * dot / (float)n;
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      const int c = tid + k * T;
+      float a[8], g[8], w[8], o[8];
+      unpack8(rx[k], a);
+      unpack8(rg[k], g);
+      unpack8(gm[k], w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        o[j] = (r * g[j]) * w[j] - coef * a[j];
+        acc[k][j] += (a[j] * g[j]) * r;
+      }
+      if (c * 8 < n) *(uint4*)(dx + row * n + c * 8) = pack8_bf16(o);
+    }
+  };
+
+  if (r0 < r1) {
+    uint4 xa[NCHUNK], ga[NCHUNK], xb[NCHUNK], gb[NCHUNK];
+    load_row<T, NCHUNK>(x + r0 * n, n, xa);
+    load_row<T, NCHUNK>(dy + r0 * n, n, ga);
+    for (int64_t row = r0; row < r1; row += 2) {
+      if (row + 1 < r1) {
+        load_row<T, NCHUNK>(x + (row + 1) * n, n, xb);
+        load_row<T, NCHUNK>(dy + (row + 1) * n, n, gb);
+      }
+      process(xa, ga, row, 0);
+      if (row + 1 < r1) {
+        if (row + 2 < r1) {
+          load_row<T, NCHUNK>(x + (row + 2) * n, n, xa);
+          load_row<T, NCHUNK>(dy + (row + 2) * n, n, ga);
+        }
+        process(xb, gb, row + 1, 1);
+      }
+    }
+  }
+  // every workgroup writes its (possibly zero) partial: the reduction reads all of them
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) {
+    const int c = tid + k * T;
+    if (c * 8 < n) {
+      float4* dst = (float4*)(dg_part + (int64_t)blockIdx.x * n + c * 8);
+      dst[0] = make_float4(acc[k][0], acc[k][1], acc[k][2], acc[k][3]);
+      dst[1] = make_float4(acc[k][4], acc[k][5], acc[k][6], acc[k][7]);
+    }
+  }
+}
+
+// dgamma[c] = sum_p part[p, c], fixed order: 4 strided slices of p summed
+// sequentially, then combined 0..3.  64 columns per workgroup.
+__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                     int P, int n) {
+  __shared__ float red[4][64];
+  const int col = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int slice = threadIdx.x >> 6;
+  float acc = 0.f;
+  if (col < n)
+    for (int p = slice; p < P; p += 4) acc += part[(int64_t)p * n + col];
+  red[slice][threadIdx.x & 63] = acc;
+  __syncthreads();
+  if (slice == 0 && col < n)
+    out[col] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+}
+
+// ---------------------------------------------------------------------------
+// row-wise 1x128 group quant of a flat run of groups (scale index == group index)
+// ---------------------------------------------------------------------------
+template <int KIND, bool ROUND>
+__global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
+                                                          float* __restrict__ s, int64_t n_groups) {
+  const int64_t g0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  const int64_t stride = ((int64_t)gridDim.x * 256) >> 4;
+  const int sub = threadIdx.x & 15;
+  const int64_t limit = (n_groups + stride - 1) / stride * stride;  // keep the 16 lanes of a row together
+  for (int64_t g = g0; g < limit; g += stride) {
+    const bool ok = g < n_groups;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (ok) raw = *(const uint4*)(x + g * kGroup + sub * 8);
+    float a[8];
+    unpack8(raw, a);
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(a[j]));
+    m = row16_max(m);
+    const float sc = make_scale<KIND, ROUND>(m);
+    const Divisor d = make_divisor(sc);
+    float qv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qv[j] = div_exact(a[j], d);
+    uint2 pk;
+    pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+    pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+    if (ok) {
+      *(uint2*)(q + g * kGroup + sub * 8) = pk;
+      if (sub == 0) s[g] = sc;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// launchers
+// ---------------------------------------------------------------------------
+// pick the workgroup width and chunks-per-thread for a row of n columns
+static void pick_row_shape(int n, int& T, int& nchunk) {
+  const int chunks = (n + 7) / 8;
+  T = 256;
+  if (chunks <= 64) T = 64;
+  else if (chunks <= 128) T = 128;
+  else if (chunks % 256 != 0 && chunks % 128 == 0 && chunks / 128 <= 8) T = 128;
+  nchunk = (chunks + T - 1) / T;
+}
+
+#define FQ_ROW_CASE(TT, NC, ...) \
+  if (T == TT && nchunk == NC) { constexpr int kT = TT; constexpr int kNC = NC; __VA_ARGS__ } else
+#define FQ_ROW_SHAPES(...)                                                                               \
+  FQ_ROW_CASE(64, 1, __VA_ARGS__) FQ_ROW_CASE(128, 1, __VA_ARGS__) FQ_ROW_CASE(128, 2, __VA_ARGS__)      \
+  FQ_ROW_CASE(128, 3, __VA_ARGS__) FQ_ROW_CASE(128, 4, __VA_ARGS__) FQ_ROW_CASE(128, 5, __VA_ARGS__)     \
+  FQ_ROW_CASE(128, 6, __VA_ARGS__) FQ_ROW_CASE(128, 7, __VA_ARGS__) FQ_ROW_CASE(128, 8, __VA_ARGS__)     \
+  FQ_ROW_CASE(256, 1, __VA_ARGS__) FQ_ROW_CASE(256, 2, __VA_ARGS__) FQ_ROW_CASE(256, 3, __VA_ARGS__)     \
+  FQ_ROW_CASE(256, 4, __VA_ARGS__) { return hipErrorInvalidValue; }
+
+hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* scale, float* rstd, int64_t M,
+                              int n, float eps, int reuse_rstd, int quant, int round_scale, int kind,
+                              hipStream_t stream) {
+  if (M == 0) return hipSuccess;
+  int T, nchunk;
+  pick_row_shape(n, T, nchunk);
+  const int rows_per_wg = 16;
+  const dim3 grid((unsigned)((M + rows_per_wg - 1) / rows_per_wg));
+#define FQ_LAUNCH_FWD(REUSE, QUANT, KINDV, ROUNDV)                                                          \
+  FQ_ROW_SHAPES(hipLaunchKernelGGL((rmsnorm_fwd_kernel<kT, kNC, REUSE, QUANT, KINDV, ROUNDV>), grid,       \
+                                   dim3(kT), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, out,   \
+                                   scale, rstd, M, n, eps, rows_per_wg);)
+  if (!quant) {
+    if (reuse_rstd) { FQ_LAUNCH_FWD(true, false, kE4M3, false) } else { FQ_LAUNCH_FWD(false, false, kE4M3, false) }
+  } else if (kind == kE5M2) {
+    if (round_scale) { FQ_LAUNCH_FWD(false, true, kE5M2, true) } else { FQ_LAUNCH_FWD(false, true, kE5M2, false) }
+  } else {
+    if (round_scale) { FQ_LAUNCH_FWD(false, true, kE4M3, true) } else { FQ_LAUNCH_FWD(false, true, kE4M3, false) }
+  }
+#undef FQ_LAUNCH_FWD
+  return hipGetLastError();
+}
+
+int64_t rmsnorm_bwd_partials(int64_t M) {
+  // one partial row of dgamma per workgroup; 512 workgroups (two per CU) at most
+  const int64_t min_rows = 8;
+  int64_t p = (M + min_rows - 1) / min_rows;
+  if (p > 512) p = 512;
+  if (p < 1) p = 1;
+  return p;
+}
+
+hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
+                              float* dgamma, float* dg_part, int64_t n_partials, int64_t M, int n, float eps,
+                              hipStream_t stream) {
+  int T, nchunk;
+  pick_row_shape(n, T, nchunk);
+  const int64_t P = n_partials;
+  const int rows_per_wg = (int)((M + P - 1) / P);
+  const dim3 grid((unsigned)P);
+#define FQ_LAUNCH_BWD(REUSE)                                                                               \
+  FQ_ROW_SHAPES(hipLaunchKernelGGL((rmsnorm_bwd_kernel<kT, kNC, REUSE>), grid, dim3(kT), 0, stream,        \
+                                   (const uint16_t*)dy, (const uint16_t*)x, (const uint16_t*)gamma, rstd,  \
+                                   (uint16_t*)dx, dg_part, M, n, eps, rows_per_wg);)
+  if (rstd) { FQ_LAUNCH_BWD(true) } else { FQ_LAUNCH_BWD(false) }
+#undef FQ_LAUNCH_BWD
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, stream, dg_part, dgamma, (int)P,
+                     n);
+  return hipGetLastError();
+}
+
+hipError_t launch_group_quant(const void* x, void* q, float* s, int64_t n_groups, int round_scale, int kind,
+                              hipStream_t stream) {
+  if (n_groups == 0) return hipSuccess;
+  int64_t wgs = (n_groups + 15) / 16;  // 16 groups per workgroup pass
+  if (wgs > 256 * 16) wgs = 256 * 16;
+  const dim3 grid((unsigned)wgs), block(256);
+#define FQ_GQ(KINDV, ROUNDV) \
+  hipLaunchKernelGGL((group_quant_kernel<KINDV, ROUNDV>), grid, block, 0, stream, (const uint16_t*)x, (uint8_t*)q, s, n_groups)
+  if (kind == kE5M2) { if (round_scale) FQ_GQ(kE5M2, true); else FQ_GQ(kE5M2, false); }
+  else if (kind == kE5M2Max448) { if (round_scale) FQ_GQ(kE5M2Max448, true); else FQ_GQ(kE5M2Max448, false); }
+  else { if (round_scale) FQ_GQ(kE4M3, true); else FQ_GQ(kE4M3, false); }
+#undef FQ_GQ
+  return hipGetLastError();
+}
+
+}  // namespace fq

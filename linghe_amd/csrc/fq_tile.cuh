@@ -1,0 +1,278 @@
+// 128x128 tile quantiser shared by every "tile" kernel of the path:
+// a workgroup owns one 128-row x 128-column tile of the (already computed, fp32)
+// matrix to be quantised and emits, in one pass,
+//   * row-wise 1x128 codes + one fp32 scale per row          (MODE 0 or 2)
+//   * column-wise 128x1 codes, transposed through LDS, + one
+//     fp32 scale per column                                   (MODE 1 or 2)
+//
+// Thread mapping (RPT = rows per thread, 8 -> 256 threads, 4 -> 512 threads):
+//   cg = tid & 15   column group: columns cg*8 .. cg*8+7 (one 128-bit bf16 load)
+//   rg = tid >> 4   row group:    rows    rg*RPT .. rg*RPT+RPT-1
+// so the 16 lanes of one DPP row share a matrix row (row amax = DPP reduction),
+// and a thread owns RPT consecutive rows of 8 columns (the transposed codes of
+// one column are RPT consecutive bytes -> one LDS store).
+#pragma once
+#include "fq_device.cuh"
+
+namespace fq {
+
+template <int RPT>
+struct TileShape {
+  static_assert(RPT == 8 || RPT == 4, "rows per thread");
+  static constexpr int kRowGroups = kGroup / RPT;
+  static constexpr int kThreads = 16 * kRowGroups;
+  static constexpr int kWaves = kThreads / 64;
+};
+
+// where the four outputs of one tile go (element offsets; see the layout
+// formulas in linghe/utils/silu.py:248-276 and :507-554)
+struct TileOut {
+  uint8_t* q;       // row-wise codes:       q[q_off + i*q_ld + c]
+  int64_t q_off;
+  int64_t q_ld;
+  float* s;         // row scales:           s[s_off + i]
+  int64_t s_off;
+  uint8_t* qt;      // transposed codes:     qt[t_off + c*t_ld + i]
+  int64_t t_off;
+  int64_t t_ld;
+  float* st;        // column scales:        st[st_off + c]
+  int64_t st_off;
+  int rows_valid;   // rows i < rows_valid exist (1..128)
+};
+
+template <int RPT>
+struct alignas(16) TileShared {
+  uint8_t t[kGroup * kGroup];                       // transposed codes, 16-byte chunks XOR-swizzled
+  float colmax[TileShape<RPT>::kWaves][kGroup];      // per-wave column amax
+  float cscale[kGroup];                              // column scales
+};
+
+// xor-16 / xor-32 lane exchange + max with the gfx950 permlane swaps
+__device__ __forceinline__ float max_across_rows(float v) {
+  uint32_t u = as_u32(v);
+  auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  float m = fmaxf(as_f32(a[0]), as_f32(a[1]));
+  u = as_u32(m);
+  auto b = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return fmaxf(as_f32(b[0]), as_f32(b[1]));
+}
+
+// store up to 16 transposed code bytes; `n` of them are valid rows
+__device__ __forceinline__ void store_t_chunk(uint8_t* dst, const uint4& v, int n) {
+  if (n <= 0) return;
+  uintptr_t a = (uintptr_t)dst;
+  if (n >= 16 && (a & 15) == 0) {
+    *(uint4*)dst = v;
+    return;
+  }
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  if ((a & 3) == 0) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      if (4 * d + 4 <= n) {
+        ((uint32_t*)dst)[d] = w[d];
+      } else {
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          if (4 * d + b < n) dst[4 * d + b] = (uint8_t)(w[d] >> (8 * b));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        if (4 * d + b < n) dst[4 * d + b] = (uint8_t)(w[d] >> (8 * b));
+  }
+}
+
+// Quantise the tile held in registers (v[s][j] = element (rg*RPT+s, cg*8+j);
+// rows >= rows_valid must hold 0).  All threads of the workgroup must call it.
+template <int KIND, bool ROUND, int MODE, int RPT, bool EXACT_DIV = true>
+__device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o,
+                                              TileShared<RPT>& sh) {
+  using Shape = TileShape<RPT>;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int cg = tid & 15;
+  const int rg = tid >> 4;
+
+  // ------------------------------------------------------------- row-wise
+  if constexpr (MODE == 0 || MODE == 2) {
+    float my_scale = 0.f;
+#pragma unroll
+    for (int s = 0; s < RPT; ++s) {
+      float m = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[s][j]));
+      m = row16_max(m);
+      const float sc = make_scale<KIND, ROUND>(m);
+      if (cg == s) my_scale = sc;
+      const Divisor d = make_divisor(sc);
+      float qv[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qv[j] = EXACT_DIV ? div_exact(v[s][j], d) : v[s][j] * d.r;
+      uint2 pk;
+      pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+      pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+      const int i = rg * RPT + s;
+      if (i < o.rows_valid) *(uint2*)(o.q + o.q_off + (int64_t)i * o.q_ld + cg * 8) = pk;
+    }
+    // lane cg < RPT of each row group stores the scale of row rg*RPT+cg:
+    // a wave writes 4*RPT consecutive floats
+    if (cg < RPT) {
+      const int i = rg * RPT + cg;
+      if (i < o.rows_valid) o.s[o.s_off + i] = my_scale;
+    }
+  }
+
+  // ---------------------------------------------------------- column-wise
+  if constexpr (MODE == 1 || MODE == 2) {
+    float cm[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float m = 0.f;
+#pragma unroll
+      for (int s = 0; s < RPT; ++s) m = fmaxf(m, fabsf(v[s][j]));
+      cm[j] = max_across_rows(m);
+    }
+    if (lane < 16) {
+      float4* dst = (float4*)&sh.colmax[wave][cg * 8];
+      dst[0] = make_float4(cm[0], cm[1], cm[2], cm[3]);
+      dst[1] = make_float4(cm[4], cm[5], cm[6], cm[7]);
+    }
+    __syncthreads();
+    if (tid < kGroup) {
+      float m = sh.colmax[0][tid];
+#pragma unroll
+      for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[w][tid]);
+      const float sc = make_scale<KIND, ROUND>(m);
+      sh.cscale[tid] = sc;
+      o.st[o.st_off + tid] = sc;
+    }
+    __syncthreads();
+    float cs[8];
+    {
+      const float4* src = (const float4*)&sh.cscale[cg * 8];
+      const float4 a = src[0], b = src[1];
+      cs[0] = a.x; cs[1] = a.y; cs[2] = a.z; cs[3] = a.w;
+      cs[4] = b.x; cs[5] = b.y; cs[6] = b.z; cs[7] = b.w;
+    }
+    // transposed codes -> LDS; byte (c, i) lives at c*128 + ((i>>4) ^ ((c>>3)&7))*16 + (i&15)
+    const int i0 = rg * RPT;
+    const int chunk = (i0 >> 4) ^ (cg & 7);
+    uint8_t* base = sh.t + chunk * 16 + (i0 & 15);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const Divisor d = make_divisor(cs[j]);
+      float qv[RPT];
+#pragma unroll
+      for (int s = 0; s < RPT; ++s) qv[s] = EXACT_DIV ? div_exact(v[s][j], d) : v[s][j] * d.r;
+      uint8_t* p = base + (cg * 8 + j) * kGroup;
+      if constexpr (RPT == 8) {
+        uint2 pk;
+        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+        *(uint2*)p = pk;
+      } else {
+        *(uint32_t*)p = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+      }
+    }
+    __syncthreads();
+    // each transposed row (one column, 128 row-bytes) leaves as 8 x 16 bytes
+    constexpr int kRowsPerPass = Shape::kThreads / 8;
+    const int ch = tid & 7;
+#pragma unroll
+    for (int k = 0; k < kGroup / kRowsPerPass; ++k) {
+      const int c = (tid >> 3) + k * kRowsPerPass;
+      const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
+      store_t_chunk(o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16, val, o.rows_valid - ch * 16);
+    }
+    __syncthreads();  // LDS is reused by a following call
+  }
+}
+
+// ---------------------------------------------------------------------------
+// per-expert tile lookup for the batched forms
+// ---------------------------------------------------------------------------
+struct ExpertTile {
+  int expert;
+  int count;            // rows of this expert
+  int rb;               // 128-row block inside the expert
+  int64_t row_start;    // first global row of the expert
+  int64_t tblock_start; // sum over previous experts of ceil(count/128)
+};
+
+struct ExpertScanShared {
+  long long wave_rows[16];
+  int wave_blocks[16];
+  ExpertTile found;
+};
+
+__device__ __forceinline__ int load_count(const void* counts, int is_i64, int e) {
+  return is_i64 ? (int)((const long long*)counts)[e] : ((const int*)counts)[e];
+}
+
+// Which expert owns the global 128-row block `blk` (blocks are numbered expert
+// after expert, ceil(count/128) per expert)?  Computed from the device-side
+// counts by a block-wide prefix scan; every thread returns the same answer.
+// An out-of-range blk (host/device counts disagree) yields expert = -1.
+template <int THREADS>
+__device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int is_i64, int n_experts,
+                                                       int blk, ExpertScanShared& sh) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  constexpr int kWaves = THREADS / 64;
+  if (tid == 0) sh.found.expert = -1;
+  long long run_rows = 0;
+  int run_blocks = 0;
+  for (int base = 0; base < n_experts; base += THREADS) {
+    const int e = base + tid;
+    const int c = (e < n_experts) ? load_count(counts, is_i64, e) : 0;
+    const int nb = (c + kGroup - 1) / kGroup;
+    long long rows = c;
+    int blocks = nb;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const long long r2 = __shfl_up(rows, d, 64);
+      const int b2 = __shfl_up(blocks, d, 64);
+      if (lane >= d) { rows += r2; blocks += b2; }
+    }
+    __syncthreads();  // previous iteration's readers are done
+    if (lane == 63) { sh.wave_rows[wave] = rows; sh.wave_blocks[wave] = blocks; }
+    __syncthreads();
+    long long rows_before = run_rows;
+    int blocks_before = run_blocks;
+    long long tot_rows = 0;
+    int tot_blocks = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const long long wr = sh.wave_rows[w];
+      const int wb = sh.wave_blocks[w];
+      if (w < wave) { rows_before += wr; blocks_before += wb; }
+      tot_rows += wr;
+      tot_blocks += wb;
+    }
+    const int excl_blocks = blocks_before + blocks - nb;
+    if (nb > 0 && blk >= excl_blocks && blk < excl_blocks + nb) {
+      ExpertTile t;
+      t.expert = e;
+      t.count = c;
+      t.rb = blk - excl_blocks;
+      t.row_start = rows_before + rows - c;
+      t.tblock_start = excl_blocks;
+      sh.found = t;
+    }
+    run_rows += tot_rows;
+    run_blocks += tot_blocks;
+    if (blk < run_blocks) break;  // uniform: found in this chunk
+  }
+  __syncthreads();
+  ExpertTile out = sh.found;
+  __syncthreads();
+  return out;
+}
+
+}  // namespace fq

@@ -1,0 +1,372 @@
+// Tile kernels: one workgroup per 128x128 output tile, a single pass over HBM.
+//   blockwise_quant      plain / per-expert          (linghe/quant/block.py:65-297)
+//   silu_quant_fwd       SwiGLU (+row weight) + quant (linghe/utils/silu.py:213-335, 467-950)
+//   silu_quant_bwd       SwiGLU backward + quant      (linghe/utils/silu.py:338-464, 1097-1393)
+//   rmsnorm_quant_tile   (x*rstd)*gamma + quant with a given rstd
+//                                                    (linghe/utils/norm.py:301-340)
+#include "fq_tile.cuh"
+#include "fq_launch.h"
+
+namespace fq {
+
+// ---------------------------------------------------------------------------
+// tile geometry
+// ---------------------------------------------------------------------------
+struct TileGeom {
+  int64_t row0;      // first global row of the tile
+  int rows_valid;
+  int cb;            // 128-column block of the input
+  int64_t s_base, s_stride;
+  int64_t t_base, t_stride;
+  int64_t st_row;
+  bool valid;
+};
+
+struct BatchArgs {
+  const void* counts;  // device, int32 or int64, [n_experts]
+  int counts_i64;
+  int n_experts;
+};
+
+// out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
+// backward's dx1|dx2)
+template <bool BATCHED, int THREADS>
+__device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out_w, const BatchArgs& b,
+                                                 ExpertScanShared& scan) {
+  TileGeom g;
+  const int id = blockIdx.x;
+  const int rbk = id / ncb;
+  g.cb = id - rbk * ncb;
+  if constexpr (!BATCHED) {
+    g.row0 = (int64_t)rbk * kGroup;
+    const int64_t left = M - g.row0;
+    g.rows_valid = left < kGroup ? (int)left : kGroup;
+    g.s_base = g.row0;
+    g.s_stride = M;
+    g.t_base = g.row0;
+    g.t_stride = M;
+    g.st_row = rbk;
+    g.valid = left > 0;
+  } else {
+    const ExpertTile et = find_expert_tile<THREADS>(b.counts, b.counts_i64, b.n_experts, rbk, scan);
+    g.valid = et.expert >= 0;
+    const int left = et.count - et.rb * kGroup;
+    g.rows_valid = left < kGroup ? left : kGroup;
+    g.row0 = et.row_start + (int64_t)et.rb * kGroup;
+    g.s_base = et.row_start * (out_w / kGroup) + (int64_t)et.rb * kGroup;
+    g.s_stride = et.count;
+    g.t_base = et.row_start * out_w + (int64_t)et.rb * kGroup;
+    g.t_stride = et.count;
+    g.st_row = et.tblock_start + et.rb;
+    if (g.row0 + g.rows_valid > M) g.valid = false;  // counts disagree with the matrix: write nothing
+  }
+  return g;
+}
+
+struct OutPtrs {
+  uint8_t* q;
+  float* s;
+  uint8_t* qt;
+  float* st;
+};
+
+// ocb: 128-column block index inside the quantised matrix of width out_w
+__device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g, int64_t out_w, int ocb) {
+  TileOut o;
+  o.q = p.q;
+  o.q_off = g.row0 * out_w + (int64_t)ocb * kGroup;
+  o.q_ld = out_w;
+  o.s = p.s;
+  o.s_off = g.s_base + (int64_t)ocb * g.s_stride;
+  o.qt = p.qt;
+  o.t_off = g.t_base + (int64_t)ocb * kGroup * g.t_stride;
+  o.t_ld = g.t_stride;
+  o.st = p.st;
+  o.st_off = g.st_row * out_w + (int64_t)ocb * kGroup;
+  o.rows_valid = g.rows_valid;
+  return o;
+}
+
+// RPT rows x 8 bf16 columns of a row-major matrix; rows >= rows_valid read as 0
+template <int RPT>
+__device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
+  const int cg = threadIdx.x & 15;
+  const int rg = threadIdx.x >> 4;
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) {
+    const int i = rg * RPT + s;
+    raw[s] = make_uint4(0, 0, 0, 0);
+    if (i < rows_valid) raw[s] = *(const uint4*)(base + (int64_t)i * ld + cg * 8);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// plain blockwise quant
+// ---------------------------------------------------------------------------
+template <int KIND, bool ROUND, int MODE, bool BATCHED>
+__global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __restrict__ x, OutPtrs out,
+                                                              int64_t M, int N, BatchArgs batch) {
+  constexpr int RPT = 8;
+  __shared__ TileShared<RPT> sh;
+  __shared__ ExpertScanShared scan;
+  const TileGeom g = resolve_tile<BATCHED, 256>(M, N / kGroup, N, batch, scan);
+  if (!g.valid) return;
+  uint4 raw[RPT];
+  load_rows<RPT>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
+  float v[RPT][8];
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
+  quantize_tile<KIND, ROUND, MODE, RPT>(v, make_out(out, g, N, g.cb), sh);
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU forward + quant.  y = (sigmoid(x1)*x1)*x2 [*w_row]   (fp32)
+// ---------------------------------------------------------------------------
+struct RowWeight {
+  const void* w;   // [M] fp32 or bf16, nullptr = unweighted
+  int is_bf16;
+};
+__device__ __forceinline__ float load_weight(const RowWeight& w, int64_t r) {
+  return w.is_bf16 ? as_f32((uint32_t)((const uint16_t*)w.w)[r] << 16) : ((const float*)w.w)[r];
+}
+
+template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED>
+__global__ __launch_bounds__(256) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
+                                                             OutPtrs out, int64_t M, int n, BatchArgs batch) {
+  constexpr int RPT = 8;
+  __shared__ TileShared<RPT> sh;
+  __shared__ ExpertScanShared scan;
+  const TileGeom g = resolve_tile<BATCHED, 256>(M, n / kGroup, n, batch, scan);
+  if (!g.valid) return;
+  const int64_t ld = 2 * (int64_t)n;
+  uint4 r1[RPT], r2[RPT];
+  const uint16_t* p = x + g.row0 * ld + (int64_t)g.cb * kGroup;
+  load_rows<RPT>(p, ld, g.rows_valid, r1);
+  load_rows<RPT>(p + n, ld, g.rows_valid, r2);
+  const int rg = threadIdx.x >> 4;
+  float v[RPT][8];
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) {
+    float a[8], b[8];
+    unpack8(r1[s], a);
+    unpack8(r2[s], b);
+    float w = 1.0f;
+    if constexpr (WEIGHTED) {
+      const int i = rg * RPT + s;
+      w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float y = (sigmoid_f32(a[j]) * a[j]) * b[j];
+      if constexpr (WEIGHTED) y = y * w;
+      v[s][j] = y;
+    }
+  }
+  quantize_tile<KIND, ROUND, MODE, RPT>(v, make_out(out, g, n, g.cb), sh);
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU backward + quant.  With h = g[*w]*x2 and sg = sigmoid(x1):
+//   dx1 = h*sg + ((h*x1)*(1-sg))*sg        dx2 = g[*w]*(sg*x1)
+//   dw_row = sum_c g*((sg*x1)*x2)          (batched form only)
+// evaluated in the order fp32 autograd evaluates them.
+// ---------------------------------------------------------------------------
+template <int KIND, bool ROUND, bool BATCHED>
+__global__ __launch_bounds__(512) void silu_quant_bwd_kernel(const uint16_t* __restrict__ gr,
+                                                             const uint16_t* __restrict__ x, RowWeight weight,
+                                                             OutPtrs out, float* __restrict__ dw_part, int64_t M,
+                                                             int n, BatchArgs batch) {
+  constexpr int RPT = 4;
+  __shared__ TileShared<RPT> sh;
+  __shared__ ExpertScanShared scan;
+  const int nb = n / kGroup;
+  const int64_t N = 2 * (int64_t)n;
+  const TileGeom g = resolve_tile<BATCHED, 512>(M, nb, N, batch, scan);
+  if (!g.valid) return;
+  uint4 r1[RPT], r2[RPT], rgd[RPT];
+  const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
+  load_rows<RPT>(p, N, g.rows_valid, r1);
+  load_rows<RPT>(p + n, N, g.rows_valid, r2);
+  load_rows<RPT>(gr + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, rgd);
+  const int cg = threadIdx.x & 15;
+  const int rg = threadIdx.x >> 4;
+  float d1[RPT][8], d2[RPT][8];
+  float my_dw = 0.f;
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) {
+    float a[8], b[8], go[8];
+    unpack8(r1[s], a);
+    unpack8(r2[s], b);
+    unpack8(rgd[s], go);
+    float w = 1.0f;
+    const int i = rg * RPT + s;
+    if constexpr (BATCHED) w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
+    float dw = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float sg = sigmoid_f32(a[j]);
+      const float sx = sg * a[j];
+      float gw = go[j];
+      if constexpr (BATCHED) {
+        dw += go[j] * (sx * b[j]);
+        gw = go[j] * w;
+      }
+      const float h = gw * b[j];
+      d2[s][j] = gw * sx;
+      d1[s][j] = h * sg + ((h * a[j]) * (1.0f - sg)) * sg;
+    }
+    if constexpr (BATCHED) {
+      dw = row16_sum(dw);
+      if (cg == s) my_dw = dw;
+    }
+  }
+  if constexpr (BATCHED) {
+    if (cg < RPT) {
+      const int i = rg * RPT + cg;
+      if (i < g.rows_valid) dw_part[(g.row0 + i) * nb + g.cb] = my_dw;
+    }
+  }
+  quantize_tile<KIND, ROUND, 2, RPT>(d1, make_out(out, g, N, g.cb), sh);
+  quantize_tile<KIND, ROUND, 2, RPT>(d2, make_out(out, g, N, nb + g.cb), sh);
+}
+
+// dw[r] = sum_b part[r, b]  (fixed order), stored as fp32 or bf16
+__global__ __launch_bounds__(256) void rowsum_kernel(const float* __restrict__ part, void* __restrict__ dw,
+                                                     int64_t M, int nb, int out_bf16) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= M) return;
+  float acc = 0.f;
+  for (int b = 0; b < nb; ++b) acc += part[r * nb + b];
+  if (out_bf16) ((uint16_t*)dw)[r] = (uint16_t)(pack_bf16x2(acc, 0.f) & 0xffffu);
+  else ((float*)dw)[r] = acc;
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm + quant on a tile with the row statistic given:
+//   y = (x * rstd[row]) * gamma[col]
+// ---------------------------------------------------------------------------
+template <int KIND, bool ROUND, int MODE>
+__global__ __launch_bounds__(256) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
+                                                                 const uint16_t* __restrict__ gamma,
+                                                                 const float* __restrict__ rstd, OutPtrs out,
+                                                                 int64_t M, int n) {
+  constexpr int RPT = 8;
+  __shared__ TileShared<RPT> sh;
+  __shared__ ExpertScanShared scan;
+  BatchArgs none{nullptr, 0, 0};
+  const TileGeom g = resolve_tile<false, 256>(M, n / kGroup, n, none, scan);
+  if (!g.valid) return;
+  uint4 raw[RPT];
+  load_rows<RPT>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
+  const int cg = threadIdx.x & 15;
+  const int rg = threadIdx.x >> 4;
+  float gm[8];
+  unpack8(*(const uint4*)(gamma + (int64_t)g.cb * kGroup + cg * 8), gm);
+  float v[RPT][8];
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) {
+    const int i = rg * RPT + s;
+    const float r = (i < g.rows_valid) ? rstd[g.row0 + i] : 0.f;
+    float a[8];
+    unpack8(raw[s], a);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[s][j] = (a[j] * r) * gm[j];
+  }
+  quantize_tile<KIND, ROUND, MODE, RPT>(v, make_out(out, g, n, g.cb), sh);
+}
+
+// ---------------------------------------------------------------------------
+// launchers
+// ---------------------------------------------------------------------------
+#define FQ_DISPATCH_BOOL(flag, NAME, ...) \
+  if (flag) { constexpr bool NAME = true; __VA_ARGS__ } else { constexpr bool NAME = false; __VA_ARGS__ }
+#define FQ_DISPATCH_KIND(kind, NAME, ...) \
+  if ((kind) == kE5M2) { constexpr int NAME = kE5M2; __VA_ARGS__ } else { constexpr int NAME = kE4M3; __VA_ARGS__ }
+#define FQ_DISPATCH_MODE(mode, NAME, ...)                                    \
+  if ((mode) == 0) { constexpr int NAME = 0; __VA_ARGS__ }                   \
+  else if ((mode) == 1) { constexpr int NAME = 1; __VA_ARGS__ }              \
+  else { constexpr int NAME = 2; __VA_ARGS__ }
+
+hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int N,
+                                  int round_scale, int mode, int kind, const void* counts, int counts_i64,
+                                  int n_experts, int64_t row_blocks, hipStream_t stream) {
+  OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
+  BatchArgs b{counts, counts_i64, n_experts};
+  const int64_t tiles = row_blocks * (N / kGroup);
+  if (tiles == 0) return hipSuccess;
+  const dim3 grid((unsigned)tiles), block(256);
+  const bool batched = counts != nullptr;
+  FQ_DISPATCH_KIND(kind, K,
+    FQ_DISPATCH_BOOL(round_scale, R,
+      FQ_DISPATCH_MODE(mode, MD,
+        FQ_DISPATCH_BOOL(batched, B,
+          hipLaunchKernelGGL((blockwise_quant_kernel<K, R, MD, B>), grid, block, 0, stream,
+                             (const uint16_t*)x, out, M, N, b);))))
+  return hipGetLastError();
+}
+
+hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_bf16, void* q, float* s, void* qt,
+                                 float* st, int64_t M, int n, int round_scale, int mode, int kind,
+                                 const void* counts, int counts_i64, int n_experts, int64_t row_blocks,
+                                 hipStream_t stream) {
+  OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
+  BatchArgs b{counts, counts_i64, n_experts};
+  RowWeight w{weight, weight_bf16};
+  const int64_t tiles = row_blocks * (n / kGroup);
+  if (tiles == 0) return hipSuccess;
+  const dim3 grid((unsigned)tiles), block(256);
+  const bool batched = counts != nullptr;
+  const bool weighted = weight != nullptr;
+  FQ_DISPATCH_KIND(kind, K,
+    FQ_DISPATCH_BOOL(round_scale, R,
+      FQ_DISPATCH_MODE(mode, MD,
+        FQ_DISPATCH_BOOL(batched, B,
+          FQ_DISPATCH_BOOL(weighted, W,
+            hipLaunchKernelGGL((silu_quant_fwd_kernel<K, R, MD, B, W>), grid, block, 0, stream,
+                               (const uint16_t*)x, w, out, M, n, b);)))))
+  return hipGetLastError();
+}
+
+hipError_t launch_silu_quant_bwd(const void* g, const void* x, const void* weight, int weight_bf16, void* q,
+                                 float* s, void* qt, float* st, float* dw_part, void* dw, int64_t M, int n,
+                                 int round_scale, int kind, const void* counts, int counts_i64, int n_experts,
+                                 int64_t row_blocks, hipStream_t stream) {
+  OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
+  BatchArgs b{counts, counts_i64, n_experts};
+  RowWeight w{weight, weight_bf16};
+  const int nb = n / kGroup;
+  const int64_t tiles = row_blocks * nb;
+  if (tiles == 0) return hipSuccess;
+  const dim3 grid((unsigned)tiles), block(512);
+  const bool batched = counts != nullptr;
+  FQ_DISPATCH_KIND(kind, K,
+    FQ_DISPATCH_BOOL(round_scale, R,
+      FQ_DISPATCH_BOOL(batched, B,
+        hipLaunchKernelGGL((silu_quant_bwd_kernel<K, R, B>), grid, block, 0, stream, (const uint16_t*)g,
+                           (const uint16_t*)x, w, out, dw_part, M, n, b);)))
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  if (batched && M > 0) {
+    hipLaunchKernelGGL(rowsum_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, stream, dw_part, dw, M, nb,
+                       weight_bf16);
+    err = hipGetLastError();
+  }
+  return err;
+}
+
+hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const float* rstd, void* q, float* s,
+                                     void* qt, float* st, int64_t M, int n, int round_scale, int mode, int kind,
+                                     hipStream_t stream) {
+  OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
+  const int64_t tiles = ((M + kGroup - 1) / kGroup) * (n / kGroup);
+  if (tiles == 0) return hipSuccess;
+  const dim3 grid((unsigned)tiles), block(256);
+  FQ_DISPATCH_KIND(kind, K,
+    FQ_DISPATCH_BOOL(round_scale, R,
+      FQ_DISPATCH_MODE(mode, MD,
+        hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD>), grid, block, 0, stream, (const uint16_t*)x,
+                           (const uint16_t*)gamma, rstd, out, M, n);)))
+  return hipGetLastError();
+}
+
+}  // namespace fq

@@ -1,0 +1,204 @@
+"""SwiGLU + blockwise-FP8 quant entry points (reference: linghe/utils/silu.py
+:279-335, :424-464, :797-950, :1293-1393).  Names, argument order, defaults,
+output tensors and scale layouts are the reference's; ``fp8_dtype`` is a
+keyword-only extension (the reference always emits e4m3fn).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+
+def _blocks_of(splits) -> int:
+    return sum((int(c) + 127) // 128 for c in splits)
+
+
+def _counts_flag(counts: torch.Tensor) -> int:
+    if counts.dtype == torch.int64:
+        return 1
+    if counts.dtype == torch.int32:
+        return 0
+    raise TypeError(f"counts must be int32 or int64, got {counts.dtype}")
+
+
+def _weight_flag(weight: torch.Tensor) -> int:
+    if weight.dtype == torch.float32:
+        return 0
+    if weight.dtype == torch.bfloat16:
+        return 1
+    raise TypeError(f"weight must be float32 or bfloat16, got {weight.dtype}")
+
+
+def triton_silu_and_block_quant_forward(
+    x, out=None, scale=None, round_scale=False, output_mode=2, *, fp8_dtype=torch.float8_e4m3fn
+):
+    """
+    fused silu and blockwise quantization, used in shared expert
+    Args:
+        x: input tensor, bf16 [M, 2n] (gate | up)
+        round_scale: whether round scale to power of 2
+        output_mode: one of {0, 1, 2}
+            0: only output non-transposed quantized tensor
+            1: only output transposed quantized tensor
+            2: output both
+
+    Returns:
+        - out: quantized tensor [M, n]
+        - scale: quantization scale [n/128, M]
+        - transpose_output: quantized tensor of transposed output [n, M]
+        - transpose_scale: quantization scale of transposed output [ceil(M/128), n]
+    """
+    assert x.is_contiguous()
+    _lib.require_device_bf16(x, "x")
+    M, N = x.shape
+    n = N // 2
+    assert output_mode in (0, 1, 2)
+    assert n % 128 == 0 and N == 2 * n
+    device = x.device
+    if out is None:
+        out = torch.empty((M, n), device=device, dtype=fp8_dtype)
+    if scale is None:
+        scale = torch.empty((n // 128, M), device=device, dtype=torch.float32)
+    transpose_output = torch.empty((n, M), device=device, dtype=fp8_dtype)
+    transpose_scale = torch.empty(((M + 127) // 128, n), device=device, dtype=torch.float32)
+    if M > 0:
+        with torch.cuda.device(device):
+            _lib.check(_lib.lib.fq_swiglu_quant_fwd(
+                _lib.ptr(x), _lib.ptr(out), _lib.ptr(scale), _lib.ptr(transpose_output),
+                _lib.ptr(transpose_scale), M, n, int(bool(round_scale)), output_mode,
+                _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
+    return out, scale, transpose_output, transpose_scale
+
+
+def triton_silu_and_block_quant_backward(g, x, round_scale=False, *, fp8_dtype=torch.float8_e4m3fn):
+    """
+    backward of triton_silu_and_block_quant_forward
+    Args:
+        g: gradient, bf16 [M, n]
+        x: input tensor, bf16 [M, 2n]
+        round_scale: whether round to power of 2
+
+    Returns:
+        - dx: quantized non-transposed gradient [M, 2n]
+        - dx_scale: scales of quantization non-transposed gradient [2n/128, M]
+        - transpose_dx: quantized transposed gradient [2n, M]
+        - transpose_dx_scale: scales of quantization transposed gradient [M/128, 2n]
+    """
+    assert g.is_contiguous()
+    assert x.is_contiguous()
+    M, N = x.shape
+    n = N // 2
+    assert M % 128 == 0 and N % 256 == 0
+    assert g.shape == (M, n)
+    _lib.require_device_bf16(x, "x")
+    _lib.require_device_bf16(g, "g")
+    device = x.device
+    dx = torch.empty((M, N), device=device, dtype=fp8_dtype)
+    dx_scale = torch.empty((N // 128, M), device=device, dtype=torch.float32)
+    transpose_dx = torch.empty((N, M), device=device, dtype=fp8_dtype)
+    transpose_dx_scale = torch.empty(((M + 127) // 128, N), device=device, dtype=torch.float32)
+    if M > 0:
+        with torch.cuda.device(device):
+            _lib.check(_lib.lib.fq_swiglu_quant_bwd(
+                _lib.ptr(g), _lib.ptr(x), _lib.ptr(dx), _lib.ptr(dx_scale), _lib.ptr(transpose_dx),
+                _lib.ptr(transpose_dx_scale), M, n, int(bool(round_scale)), _lib.fp8_kind(fp8_dtype),
+                _lib.stream_of(x)))
+    return dx, dx_scale, transpose_dx, transpose_dx_scale
+
+
+def triton_batch_weighted_silu_and_block_quant_forward(
+    x,
+    weight,
+    counts,
+    splits=None,
+    out=None,
+    scale=None,
+    round_scale=False,
+    output_mode=2,
+    *,
+    fp8_dtype=torch.float8_e4m3fn,
+):
+    """
+    silu and blockwise quantize activation in routed experts
+    Args:
+        x: activation tensor in routed experts, bf16 [M, 2n]
+        weight: router prob tensor [M, 1]
+        counts: device tensor of token count per expert
+        splits: python int list of token count per expert
+        round_scale: whether round scale to power of 2
+        output_mode: one of {0, 1, 2}
+
+    Returns (per-expert packed layouts):
+        - out: quantized tensor [M, n]
+        - scale: per expert [n/128, count_e] blocks, allocated [M, n/128]
+        - transpose_output: per expert [n, count_e] blocks, allocated [M, n]
+        - transpose_scale: [sum ceil(count_e/128), n]
+    """
+    assert splits is not None, "batch mode need splits to launch kernels"
+    assert x.is_contiguous() and weight.is_contiguous()
+    _lib.require_device_bf16(x, "x")
+    M, N = x.shape
+    n = N // 2
+    n_experts = counts.shape[0]
+    assert N <= 8192
+    assert n % 128 == 0 and N == 2 * n
+    assert output_mode in (0, 1, 2)
+    assert weight.numel() == M
+    device = x.device
+    if out is None:
+        out = torch.empty((M, n), device=device, dtype=fp8_dtype)
+    if scale is None:
+        scale = torch.empty((M, n // 128), device=device, dtype=torch.float32)
+    blocks = _blocks_of(splits)
+    transpose_output = torch.empty((M, n), device=device, dtype=fp8_dtype)
+    transpose_scale = torch.empty((blocks, n), device=device, dtype=torch.float32)
+    if M == 0:
+        return out, scale, transpose_output, transpose_scale
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib.fq_batched_swiglu_quant_fwd(
+            _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(counts), _counts_flag(counts),
+            n_experts, blocks, _lib.ptr(out), _lib.ptr(scale), _lib.ptr(transpose_output),
+            _lib.ptr(transpose_scale), M, n, int(bool(round_scale)), output_mode,
+            _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
+    return out, scale, transpose_output, transpose_scale
+
+
+def triton_batch_weighted_silu_and_block_quant_backward(
+    g, x, weight, counts, splits=None, round_scale=False, *, fp8_dtype=torch.float8_e4m3fn
+):
+    """
+    backward of triton_batch_weighted_silu_and_block_quant_forward
+    Returns:
+        - dx: quantized non-transposed gradient [M, 2n]
+        - dx_scale: per-expert packed scales, allocated [M, 2n/128]
+        - dw: gradient of weight, shape and dtype of weight
+        - transpose_dx: per-expert packed transposed gradient, allocated [M, 2n]
+        - transpose_dx_scale: [sum ceil(count_e/128), 2n]
+    """
+    M, N = x.shape
+    n = N // 2
+    n_expert = counts.shape[0]
+    assert n % 128 == 0
+    assert g.is_contiguous()
+    assert x.is_contiguous() and weight.is_contiguous()
+    assert splits is not None, "batch mode need splits to launch kernels"
+    _lib.require_device_bf16(x, "x")
+    _lib.require_device_bf16(g, "g")
+    device = x.device
+    dx = torch.empty((M, N), device=device, dtype=fp8_dtype)
+    dx_scale = torch.empty((M, N // 128), device=device, dtype=torch.float32)
+    s = _blocks_of(splits)
+    transpose_dx = torch.empty((M, N), device=device, dtype=fp8_dtype)
+    transpose_dx_scale = torch.empty((s, N), device=device, dtype=torch.float32)
+    dw = torch.empty_like(weight)
+    if s == 0:
+        return dx, dx_scale, dw, transpose_dx, transpose_dx_scale
+    dws = torch.empty((M, n // 128), device=device, dtype=torch.float32)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib.fq_batched_swiglu_quant_bwd(
+            _lib.ptr(g), _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(counts),
+            _counts_flag(counts), n_expert, s, _lib.ptr(dx), _lib.ptr(dx_scale), _lib.ptr(dw),
+            _lib.ptr(transpose_dx), _lib.ptr(transpose_dx_scale), _lib.ptr(dws), M, n,
+            int(bool(round_scale)), _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
+    return dx, dx_scale, dw, transpose_dx, transpose_dx_scale

@@ -1,0 +1,121 @@
+"""Acceptance rules used by the parity tests (TEST INFRASTRUCTURE ONLY).
+
+* scales: distance in units in the last place, through the int32 view of the
+  positive fp32 values;
+* FP8 codes: fraction of bit-identical codes and the largest distance in code
+  steps (codes are mapped to a monotone integer line, so +0/-0 are 0 apart and
+  neighbours are 1 apart);
+* dequantisation bound: |q*s - v| <= half a code step at q's exponent, times s;
+* ``output_check_like``: the reference's own, looser, elementwise rule
+  (linghe/tools/check.py:11-129: |d| < rtol*|ref| + atol after upcasting).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+
+def ulp_distance(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Elementwise distance in fp32 ulps (both finite, same sign expected)."""
+    ai = a.detach().float().contiguous().view(torch.int32).to(torch.int64)
+    bi = b.detach().float().contiguous().view(torch.int32).to(torch.int64)
+    # map the sign-magnitude pattern to a monotone line
+    ai = torch.where(ai < 0, -(ai & 0x7FFFFFFF), ai)
+    bi = torch.where(bi < 0, -(bi & 0x7FFFFFFF), bi)
+    return (ai - bi).abs()
+
+
+def code_line(codes: torch.Tensor) -> torch.Tensor:
+    """fp8 bit patterns (any fp8 dtype or uint8) -> signed monotone integers."""
+    u = codes.detach().contiguous().view(torch.uint8).to(torch.int32)
+    mag = u & 0x7F
+    return torch.where(u >= 128, -mag, mag)
+
+
+@dataclass
+class CodeReport:
+    total: int
+    identical: int
+    max_step: int
+
+    @property
+    def identical_frac(self) -> float:
+        return 1.0 if self.total == 0 else self.identical / self.total
+
+
+def compare_codes(ref: torch.Tensor, got: torch.Tensor) -> CodeReport:
+    assert ref.shape == got.shape, (ref.shape, got.shape)
+    if ref.numel() == 0:
+        return CodeReport(0, 0, 0)
+    d = (code_line(ref) - code_line(got)).abs()
+    return CodeReport(int(d.numel()), int((d == 0).sum()), int(d.max()))
+
+
+@dataclass
+class ScaleReport:
+    total: int
+    exact: int
+    within_1ulp: int
+    max_ulp: int
+
+
+def compare_scales(ref: torch.Tensor, got: torch.Tensor) -> ScaleReport:
+    assert ref.shape == got.shape, (ref.shape, got.shape)
+    if ref.numel() == 0:
+        return ScaleReport(0, 0, 0, 0)
+    d = ulp_distance(ref, got)
+    return ScaleReport(int(d.numel()), int((d == 0).sum()), int((d <= 1).sum()), int(d.max()))
+
+
+def assert_codes(ref, got, name="codes", min_identical=0.9999, max_step=1):
+    rep = compare_codes(ref, got)
+    assert rep.identical_frac >= min_identical and rep.max_step <= max_step, (
+        f"{name}: identical {rep.identical}/{rep.total} "
+        f"({rep.identical_frac:.6f}), max step {rep.max_step}")
+    return rep
+
+
+def assert_scales(ref, got, name="scales", max_ulp=1, min_within_1ulp=1.0):
+    rep = compare_scales(ref, got)
+    frac = 1.0 if rep.total == 0 else rep.within_1ulp / rep.total
+    assert rep.max_ulp <= max_ulp and frac >= min_within_1ulp, (
+        f"{name}: exact {rep.exact}/{rep.total}, <=1ulp {rep.within_1ulp}, "
+        f"max {rep.max_ulp} ulp")
+    return rep
+
+
+def fp8_half_step(q: torch.Tensor, fp8_dtype) -> torch.Tensor:
+    """Half the spacing of the fp8 grid at the value q (fp32 tensor of decoded
+    codes).  e4m3: 3 mantissa bits, min normal exponent -6; e5m2: 2 bits, -14."""
+    mant, emin = (3, -6) if fp8_dtype == torch.float8_e4m3fn else (2, -14)
+    a = q.abs().clamp_min(2.0 ** emin)
+    e = torch.floor(torch.log2(a))
+    return torch.exp2(e - mant - 1)
+
+
+def assert_dequant_bound(values, codes, scales_per_elem, fp8_dtype, name="dequant",
+                         slack=1.0 + 2.0 ** -12):
+    """|decode(code)*s - v| <= half a code step * s (small slack for the fp32
+    rounding of the quotient)."""
+    q = codes.float().double()
+    s = scales_per_elem.double()
+    err = (q * s - values.double()).abs()
+    # at a power of two the grid below is finer than above, so the half step
+    # taken at q's own exponent bounds both sides
+    bound = fp8_half_step(q.float(), fp8_dtype).double() * s * slack
+    bad = err > bound
+    assert not bool(bad.any()), f"{name}: {int(bad.sum())} elements outside the quantisation bound"
+
+
+def output_check_like(ref, got, rtol=None, atol=None):
+    """The reference's elementwise acceptance (linghe/tools/check.py:43-69,114)."""
+    assert ref.dtype == got.dtype and ref.shape == got.shape
+    dt = ref.dtype
+    defaults = {torch.float32: (1e-4, 1e-6), torch.bfloat16: (2e-2, 1e-3),
+                torch.float8_e4m3fn: (0.125, 0.125), torch.float8_e5m2: (0.25, 0.25)}
+    r, a = defaults[dt]
+    rtol = r if rtol is None else rtol
+    atol = a if atol is None else atol
+    rf, gf = ref.float(), got.float()
+    return int(((rf - gf).abs() >= rtol * rf.abs() + atol).sum())

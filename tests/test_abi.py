@@ -1,0 +1,132 @@
+"""CPU checks of the drop-in boundary: the shared library loads and exports every
+symbol include/fq_api.h declares (no compute is launched), the Python entry
+points keep the reference's signatures, and host-side argument checks fire
+before anything reaches a device."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fq_api.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from linghe_amd import _lib
+
+    names = declared_symbols()
+    assert len(names) >= 13
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in names:
+        assert hasattr(raw, name), f"{name} declared in fq_api.h but not exported"
+    bound = set(_lib.SIGNATURES) | set(_lib.OTHER_SYMBOLS)
+    assert bound == set(names), bound ^ set(names)
+    assert _lib.lib.fq_version() >= 100
+
+
+def test_argument_counts_match_header():
+    from linghe_amd import _lib
+
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    for name, argtypes in _lib.SIGNATURES.items():
+        m = re.search(r"\b" + name + r"\s*\((.*?)\)\s*;", text, flags=re.S)
+        assert m, name
+        n_args = len([a for a in m.group(1).split(",") if a.strip()])
+        assert n_args == len(argtypes), (name, n_args, len(argtypes))
+
+
+def test_c_side_validation_without_gpu():
+    """Shape / flag errors are reported by return code before any HIP call."""
+    from linghe_amd import _lib
+
+    L = _lib.lib
+    # width not a multiple of 128
+    rc = L.fq_blockwise_quant(None, None, None, None, None, 16, 100, 0, 2, 0, None)
+    assert rc == -2 and b"128" in L.fq_last_error()
+    # bad mode
+    rc = L.fq_swiglu_quant_fwd(None, None, None, None, None, 16, 128, 0, 7, 0, None)
+    assert rc == -1
+    # NULL outputs
+    rc = L.fq_blockwise_quant(None, None, None, None, None, 16, 128, 0, 2, 0, None)
+    assert rc == -1
+    # unknown fp8 kind
+    rc = L.fq_group_quant(None, None, None, 16, 128, 0, 9, None)
+    assert rc == -1
+    # hidden size too large for the row kernels
+    rc = L.fq_rmsnorm_fwd(None, None, None, None, 4, 16384, 1e-6, 0, None)
+    assert rc == -2
+    # empty problem is a no-op
+    assert L.fq_group_quant(None, None, None, 0, 128, 0, 0, None) == 0
+    with pytest.raises(RuntimeError):
+        _lib.check(-2)
+
+
+REFERENCE_SIGNATURES = {
+    # reference file:line -> (module, function, parameter names in order)
+    "linghe/utils/norm.py:58": ("linghe_amd.utils.norm", "triton_rms_norm_forward",
+                                ["x", "weight", "eps", "out", "rms"]),
+    "linghe/utils/norm.py:144": ("linghe_amd.utils.norm", "triton_rms_norm_backward",
+                                 ["grad_output", "x", "w", "eps", "rms"]),
+    "linghe/utils/norm.py:343": ("linghe_amd.utils.norm", "triton_rms_norm_and_block_quant_forward",
+                                 ["x", "weight", "eps", "out", "scale", "rms", "round_scale", "output_mode"]),
+    "linghe/utils/silu.py:279": ("linghe_amd.utils.silu", "triton_silu_and_block_quant_forward",
+                                 ["x", "out", "scale", "round_scale", "output_mode"]),
+    "linghe/utils/silu.py:424": ("linghe_amd.utils.silu", "triton_silu_and_block_quant_backward",
+                                 ["g", "x", "round_scale"]),
+    "linghe/utils/silu.py:797": ("linghe_amd.utils.silu", "triton_batch_weighted_silu_and_block_quant_forward",
+                                 ["x", "weight", "counts", "splits", "out", "scale", "round_scale", "output_mode"]),
+    "linghe/utils/silu.py:1293": ("linghe_amd.utils.silu", "triton_batch_weighted_silu_and_block_quant_backward",
+                                  ["g", "x", "weight", "counts", "splits", "round_scale"]),
+    "linghe/quant/block.py:129": ("linghe_amd.quant.block", "triton_blockwise_quant",
+                                  ["x", "round_scale", "output_mode"]),
+    "linghe/quant/block.py:251": ("linghe_amd.quant.block", "triton_batch_blockwise_quant",
+                                  ["xs", "token_count_per_expert", "splits", "round_scale"]),
+    "linghe/quant/group.py:40": ("linghe_amd.quant.group", "triton_group_quant",
+                                 ["x", "dtype", "group_size", "round_scale"]),
+}
+
+
+@pytest.mark.parametrize("ref", sorted(REFERENCE_SIGNATURES))
+def test_entry_points_keep_reference_signatures(ref):
+    import importlib
+
+    mod, fn, params = REFERENCE_SIGNATURES[ref]
+    f = getattr(importlib.import_module(mod), fn)
+    sig = inspect.signature(f)
+    positional = [p.name for p in sig.parameters.values() if p.kind == p.POSITIONAL_OR_KEYWORD]
+    assert positional == params, (ref, positional)
+    extras = [p.name for p in sig.parameters.values() if p.kind == p.KEYWORD_ONLY]
+    assert set(extras) <= {"fp8_dtype"}
+
+
+def test_host_asserts_fire_on_cpu_tensors():
+    """Reference assert conditions are checked in Python before the library is
+    called, and CPU tensors are refused (there is no CPU path)."""
+    import torch
+
+    from linghe_amd.quant.block import triton_blockwise_quant
+    from linghe_amd.utils.silu import (triton_batch_weighted_silu_and_block_quant_forward,
+                                       triton_silu_and_block_quant_backward)
+
+    x = torch.zeros(32, 256, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        triton_blockwise_quant(x)
+    with pytest.raises(AssertionError):
+        triton_blockwise_quant(torch.zeros(17, 256, dtype=torch.bfloat16))  # M % 16
+    with pytest.raises(AssertionError):
+        triton_blockwise_quant(x.t())  # not contiguous
+    with pytest.raises(AssertionError, match="splits"):
+        triton_batch_weighted_silu_and_block_quant_forward(x, torch.zeros(32, 1), torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(AssertionError):
+        # M % 128 != 0 for the single-matrix backward
+        triton_silu_and_block_quant_backward(torch.zeros(32, 128, dtype=torch.bfloat16).cuda()
+                                             if torch.cuda.is_available() else
+                                             torch.zeros(32, 128, dtype=torch.bfloat16), x)

@@ -1,0 +1,292 @@
+"""GPU parity tests: every entry point of the hot path, called as the reference's
+own tests call theirs (tests/test_norm.py, tests/test_silu.py,
+tests/test_blockwise_quant.py, tests/test_group_quant.py of the reference),
+compared with the CPU oracle on identical seeded inputs.
+
+Acceptance (stricter than the reference's output_check):
+  * FP8 codes: >= 99.99 % bit-identical, every mismatch exactly one code step;
+  * fp32 scales: within 1 ulp.  For the fused ops the value whose amax makes the
+    scale is itself the result of fp32 arithmetic whose last bit depends on the
+    reduction order / the exp implementation, and dividing by 448 can turn a
+    1-ulp difference of amax into 2 ulps of scale (the quotient's mantissa is
+    8/7 of the dividend's): there the rule is ">= 99 % within 1 ulp, none beyond
+    SCALE_SLACK_ULP";
+  * bf16 outputs: within one bf16 ulp, >= 99.9 % identical.
+"""
+import pytest
+import torch
+
+from oracle import compare as C
+from oracle import fq_oracle as O
+from tests.helpers import (E4M3, E5M2, announce, check_quant_pair, gamma_bf16, gen, randn_bf16,
+                           zipf_counts)
+
+pytestmark = pytest.mark.gpu
+
+SCALE_SLACK_ULP = 4
+FUSED = dict(scale_max_ulp=SCALE_SLACK_ULP, scale_min_within1=0.99)
+
+
+def _dev(t, gpu):
+    return t.to(gpu)
+
+
+def check_bf16(name, ref, got, min_identical=0.999):
+    got = got.detach().cpu()
+    assert ref.dtype == got.dtype == torch.bfloat16 and ref.shape == got.shape
+    a = ref.view(torch.int16).to(torch.int32)
+    b = got.view(torch.int16).to(torch.int32)
+    a = torch.where(a < 0, -(a & 0x7FFF), a)
+    b = torch.where(b < 0, -(b & 0x7FFF), b)
+    d = (a - b).abs()
+    frac = float((d == 0).float().mean()) if d.numel() else 1.0
+    print(f"[parity] {name}: bf16 identical {frac:.6f}, max {int(d.max()) if d.numel() else 0} ulp", flush=True)
+    assert frac >= min_identical and (d.numel() == 0 or int(d.max()) <= 1), (name, frac, int(d.max()))
+
+
+# ------------------------------------------------------------------ plain quantisers
+@pytest.mark.parametrize("M,N", [(256, 256), (4096, 2048), (2064, 1536)])
+@pytest.mark.parametrize("round_scale", [False, True])
+def test_blockwise_quant(gpu, M, N, round_scale):
+    from linghe_amd.quant.block import triton_blockwise_quant
+
+    announce("blockwise_quant", M, N, round_scale)
+    x = randn_bf16(gen(11), M, N)
+    ref = O.blockwise_quant(x, round_scale)
+    xd = _dev(x, gpu)
+    for mode in (2, 0, 1):
+        q, s, qt, st = triton_blockwise_quant(xd, round_scale=round_scale, output_mode=mode)
+        torch.cuda.synchronize()
+        assert q.shape == (M, N) and s.shape == (N // 128, M)
+        assert qt.shape == (N, M) and st.shape == ((M + 127) // 128, N)
+        if mode != 1:
+            check_quant_pair(f"blockwise.m{mode}.row", ref[0], ref[1], q, s, scale_max_ulp=0, min_identical=1.0)
+        if mode != 0:
+            check_quant_pair(f"blockwise.m{mode}.col", ref[2], ref[3], qt, st, scale_max_ulp=0, min_identical=1.0)
+
+
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+def test_blockwise_quant_dequant_bound(gpu, dtype):
+    from linghe_amd.quant.block import triton_blockwise_quant
+
+    announce("blockwise_quant dequant bound", dtype)
+    M, N = 512, 384
+    x = randn_bf16(gen(12), M, N, scale=3.0)
+    x[5, 7] = 200.0  # outlier
+    q, s, qt, st = triton_blockwise_quant(_dev(x, gpu), fp8_dtype=dtype)
+    torch.cuda.synchronize()
+    q, s, qt, st = q.cpu(), s.cpu(), qt.cpu(), st.cpu()
+    xf = x.float()
+    C.assert_dequant_bound(xf, q, s.t().repeat_interleave(128, 1), dtype, "row")
+    C.assert_dequant_bound(xf.t(), qt, st.t().repeat_interleave(128, 1)[:, :M], dtype, "col")
+    ref = O.blockwise_quant(x, False, dtype)
+    check_quant_pair("blockwise.%s.row" % dtype, ref[0], ref[1], q, s, scale_max_ulp=0, min_identical=1.0)
+    check_quant_pair("blockwise.%s.col" % dtype, ref[2], ref[3], qt, st, scale_max_ulp=0, min_identical=1.0)
+    # the amax element of every group is the largest code
+    fmax = O.fp8_max(dtype)
+    assert float(q.float().abs().reshape(M, N // 128, 128).amax(2).min()) == fmax
+
+
+@pytest.mark.parametrize("M,N", [(2049, 2048), (64, 128), (1000, 8192 + 128)])
+@pytest.mark.parametrize("round_scale", [False, True])
+def test_group_quant(gpu, M, N, round_scale):
+    from linghe_amd.quant.group import triton_group_quant
+
+    announce("group_quant", M, N, round_scale)
+    x = randn_bf16(gen(13), M, N)
+    rq, rs = O.group_quant_1x128(x, round_scale)
+    q, s = triton_group_quant(_dev(x, gpu), round_scale=round_scale)
+    torch.cuda.synchronize()
+    assert s.shape == (M, N // 128)
+    check_quant_pair("group", rq, rs, q, s, scale_max_ulp=0, min_identical=1.0)
+    # e5m2 codes on the 448-based scale, as the reference kernel does
+    q5, s5 = triton_group_quant(_dev(x, gpu), dtype=E5M2, round_scale=round_scale)
+    torch.cuda.synchronize()
+    ref5 = (x.float().reshape(M, N // 128, 128) / rs.unsqueeze(-1)).to(E5M2).reshape(M, N)
+    check_quant_pair("group.e5m2", ref5, rs, q5, s5, scale_max_ulp=0, min_identical=1.0)
+
+
+@pytest.mark.parametrize("counts", [[128, 0, 256, 16, 0, 144, 1, 127], [0, 0, 0, 0], [300],
+                                    [33, 65, 7, 129, 513, 2, 0, 90, 128, 128, 77, 5, 0, 0, 250, 31]])
+def test_batch_blockwise_quant(gpu, counts):
+    from linghe_amd.quant.block import triton_batch_blockwise_quant
+
+    announce("batch_blockwise_quant", counts)
+    M, N = sum(counts), 384
+    x = randn_bf16(gen(14), M, N)
+    ref = O.batch_blockwise_quant(x, counts, False)
+    for cdt in (torch.int32, torch.int64):
+        cnt = torch.tensor(counts, dtype=cdt, device=gpu)
+        q, s, qt, st = triton_batch_blockwise_quant(_dev(x, gpu), cnt, counts)
+        torch.cuda.synchronize()
+        assert s.shape == (M * N // 128,) and qt.shape == (M * N,)
+        if M == 0:
+            continue
+        check_quant_pair("batch_blockwise.row", ref[0], ref[1], q, s, scale_max_ulp=0, min_identical=1.0)
+        check_quant_pair("batch_blockwise.col", ref[2], ref[3], qt, st, scale_max_ulp=0, min_identical=1.0)
+
+
+# ------------------------------------------------------------------ RMSNorm
+@pytest.mark.parametrize("M,N", [(1024, 2048), (1024, 1664), (208, 1664), (512, 4096), (256, 8192),
+                                 (300, 512), (64, 7168), (130, 1536)])
+def test_rmsnorm_fwd_bwd(gpu, M, N):
+    """reference tests/test_norm.py:114-145 (inputs randn**3, weight randn)."""
+    from linghe_amd.utils.norm import triton_rms_norm_backward, triton_rms_norm_forward
+
+    announce("rmsnorm fwd/bwd", M, N)
+    g = gen(21)
+    x = (torch.randn(M, N, generator=g) ** 3).to(torch.bfloat16)
+    w = torch.randn(N, generator=g).to(torch.bfloat16)
+    dy = torch.randn(M, N, generator=g).to(torch.bfloat16)
+    y_ref, r_ref = O.rms_norm_forward(x, w)
+    xd, wd, dyd = _dev(x, gpu), _dev(w, gpu), _dev(dy, gpu)
+    y, rms = triton_rms_norm_forward(xd, wd)
+    torch.cuda.synchronize()
+    check_bf16("rmsnorm.y", y_ref, y)
+    C.assert_scales(r_ref, rms.cpu(), "rstd", max_ulp=2, min_within_1ulp=0.99)
+    y2, _ = triton_rms_norm_forward(xd, wd, rms=rms)
+    torch.cuda.synchronize()
+    assert torch.equal(y2.cpu(), y.cpu())
+    dx_ref, dw_ref = O.rms_norm_backward(x, w, dy)
+    dx, dw = triton_rms_norm_backward(dyd, xd, wd)
+    torch.cuda.synchronize()
+    assert dw.dtype == torch.float32 and dw.shape == (N,)
+    check_bf16("rmsnorm.dx", dx_ref, dx, min_identical=0.995)
+    torch.testing.assert_close(dw.cpu(), dw_ref, rtol=2e-4, atol=2e-4 * float(dw_ref.abs().max()))
+    dx2, dw2 = triton_rms_norm_backward(dyd, xd, wd, rms=rms)
+    torch.cuda.synchronize()
+    assert torch.equal(dx2.cpu(), dx.cpu()) and torch.equal(dw2.cpu(), dw.cpu())
+    # 3-D input
+    if M % 4 == 0:
+        y3, _ = triton_rms_norm_forward(xd.view(4, M // 4, N), wd)
+        torch.cuda.synchronize()
+        assert y3.shape == (4, M // 4, N) and torch.equal(y3.view(M, N).cpu(), y.cpu())
+
+
+@pytest.mark.parametrize("M,N", [(1024, 2048), (2048, 1536), (200, 512), (136, 7168), (128, 128)])
+@pytest.mark.parametrize("round_scale", [True, False])
+def test_rmsnorm_and_block_quant(gpu, M, N, round_scale):
+    """reference tests/test_norm.py:189-220 (x = randn**2, weight randn, modes 0, 1, 2)."""
+    from linghe_amd.utils.norm import triton_rms_norm_and_block_quant_forward as fwd
+
+    announce("rmsnorm+quant", M, N, round_scale)
+    g = gen(22)
+    x = (torch.randn(M, N, generator=g) ** 2).to(torch.bfloat16)
+    w = torch.randn(N, generator=g).to(torch.bfloat16)
+    q_ref, s_ref, r_ref, qt_ref, st_ref = O.rms_norm_and_block_quant_forward(x, w, round_scale=round_scale)
+    xd, wd = _dev(x, gpu), _dev(w, gpu)
+    kw = dict(FUSED)
+    if round_scale:
+        kw = dict(scale_max_ulp=0, scale_min_within1=1.0)  # power-of-two scales absorb the last-bit noise
+    q, s, rms, qt0, st0 = fwd(xd, wd, round_scale=round_scale, output_mode=0)
+    torch.cuda.synchronize()
+    assert qt0.shape == (N, M) and st0.shape == ((M + 127) // 128, N)
+    check_quant_pair("rms.0.row", q_ref, s_ref, q, s, **kw)
+    C.assert_scales(r_ref, rms.cpu(), "rstd", max_ulp=2, min_within_1ulp=0.99)
+    o1, s1, rms1, qt, st = fwd(xd, wd, round_scale=round_scale, rms=rms, output_mode=1)
+    torch.cuda.synchronize()
+    assert o1 is None and s1 is None and rms1 is rms
+    check_quant_pair("rms.1.col", qt_ref, st_ref, qt, st, **kw)
+    q, s, rms2, qt, st = fwd(xd, wd, round_scale=round_scale, output_mode=2)
+    torch.cuda.synchronize()
+    assert torch.equal(rms2.cpu(), rms.cpu())
+    check_quant_pair("rms.2.row", q_ref, s_ref, q, s, **kw)
+    check_quant_pair("rms.2.col", qt_ref, st_ref, qt, st, **kw)
+
+
+# ------------------------------------------------------------------ SwiGLU
+@pytest.mark.parametrize("M,N,coef", [(2048, 1024, 1.0), (1024, 4096, 1.0), (1000, 1536, 1.0),
+                                      (512, 1536 * 8, 100.0), (512, 1536 * 8, 0.0)])
+def test_silu_and_block_quant_fwd(gpu, M, N, coef):
+    """reference tests/test_silu.py:405-436."""
+    from linghe_amd.utils.silu import triton_silu_and_block_quant_forward as fwd
+
+    announce("silu+quant fwd", M, N, coef)
+    x = randn_bf16(gen(31), M, N, scale=coef)
+    ref = O.silu_and_block_quant_forward(x, False)
+    xd = _dev(x, gpu)
+    for mode in (0, 1, 2):
+        q, s, qt, st = fwd(xd, round_scale=False, output_mode=mode)
+        torch.cuda.synchronize()
+        if mode != 1:
+            check_quant_pair(f"silu.{mode}.row", ref[0], ref[1], q, s, **FUSED)
+        if mode != 0:
+            check_quant_pair(f"silu.{mode}.col", ref[2], ref[3], qt, st, **FUSED)
+
+
+@pytest.mark.parametrize("M,N,coef,gcoef", [(2048, 1024, 1.0, 1.0), (1024, 4096, 1.0, 1e-3),
+                                            (512, 1536 * 8, 100.0, 100.0), (512, 1536 * 8, 0.0, 0.0)])
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+def test_silu_and_block_quant_bwd(gpu, M, N, coef, gcoef, dtype):
+    """reference tests/test_silu.py:437-446; e5m2 is this build's extension."""
+    from linghe_amd.utils.silu import triton_silu_and_block_quant_backward as bwd
+
+    announce("silu+quant bwd", M, N, coef, gcoef, dtype)
+    g = gen(32)
+    x = randn_bf16(g, M, N, scale=coef)
+    dy = randn_bf16(g, M, N // 2, scale=gcoef)
+    ref = O.silu_and_block_quant_backward(dy, x, False, dtype)
+    dq, ds, dqt, dst = bwd(_dev(dy, gpu), _dev(x, gpu), round_scale=False, fp8_dtype=dtype)
+    torch.cuda.synchronize()
+    assert dq.shape == (M, N) and ds.shape == (N // 128, M) and dqt.shape == (N, M) and dst.shape == (M // 128, N)
+    assert dq.dtype == dtype
+    check_quant_pair("silu.bwd.row", ref[0], ref[1], dq, ds, **FUSED)
+    check_quant_pair("silu.bwd.col", ref[2], ref[3], dqt, dst, **FUSED)
+
+
+def _batched_case(gpu, counts, N, coef, gcoef, seed, wdtype=torch.float32):
+    from linghe_amd.utils.silu import (triton_batch_weighted_silu_and_block_quant_backward as bwd,
+                                       triton_batch_weighted_silu_and_block_quant_forward as fwd)
+
+    bs = sum(counts)
+    g = gen(seed)
+    x = randn_bf16(g, bs, N, scale=coef)
+    if bs > 3:
+        x[:3] = 0.0
+    w = torch.randn(bs, 1, generator=g).to(wdtype)
+    dy = randn_bf16(g, bs, N // 2, scale=gcoef)
+    cnt = torch.tensor(counts, dtype=torch.int32, device=gpu)
+    ref = O.batch_weighted_silu_and_block_quant_forward(x, w, counts, False)
+    xd, wd, dyd = _dev(x, gpu), _dev(w, gpu), _dev(dy, gpu)
+    for mode in (2, 0, 1):
+        q, s, qt, st = fwd(xd, wd, cnt, counts, round_scale=False, output_mode=mode)
+        torch.cuda.synchronize()
+        assert q.shape == (bs, N // 2) and s.shape == (bs, N // 256) and qt.shape == (bs, N // 2)
+        if bs == 0:
+            continue
+        if mode != 1:
+            check_quant_pair(f"batch.{mode}.row", ref[0], ref[1], q, s.view(-1), **FUSED)
+        if mode != 0:
+            check_quant_pair(f"batch.{mode}.col", ref[2], ref[3], qt.view(-1), st.view(-1), **FUSED)
+    rb = O.batch_weighted_silu_and_block_quant_backward(dy, x, w, counts, False)
+    dq, ds, dw, dqt, dst = bwd(dyd, xd, wd, cnt, splits=counts, round_scale=False)
+    torch.cuda.synchronize()
+    assert dq.shape == (bs, N) and dw.shape == w.shape and dw.dtype == w.dtype
+    if bs == 0:
+        return
+    check_quant_pair("batch.bwd.row", rb[0], rb[1], dq, ds.view(-1), **FUSED)
+    check_quant_pair("batch.bwd.col", rb[3], rb[4], dqt.view(-1), dst.view(-1), **FUSED)
+    tol = 2e-2 if wdtype == torch.bfloat16 else 1e-4
+    torch.testing.assert_close(dw.cpu().float(), rb[2].float(), rtol=tol,
+                               atol=tol * max(float(rb[2].abs().max()), 1e-30))
+
+
+@pytest.mark.parametrize("counts,N,coef,gcoef", [
+    ([0] * 8, 1536, 1.0, 1.0),
+    ([160, 96, 0, 272, 16, 128, 0, 64], 1024, 1.0, 1.0),
+    ([144, 80, 400, 16], 1536, 100.0, 100.0),
+    ([144, 80, 400, 16], 1536, 0.0, 0.0),
+    ([37, 0, 129, 1, 255, 3], 512, 1.0, 1e-3),   # counts that are not multiples of 16
+    ([64, 64], 8192, 1.0, 1.0),
+])
+def test_batch_weighted_silu_and_block_quant(gpu, counts, N, coef, gcoef):
+    """reference tests/test_silu.py:588-649 (counts multiples of 16, first 3 rows zero,
+    fp32 [bs,1] weights) plus ragged counts."""
+    announce("batched silu+quant", counts, N, coef, gcoef)
+    _batched_case(gpu, counts, N, coef, gcoef, seed=33)
+
+
+def test_batch_weighted_silu_bf16_weight_many_experts(gpu):
+    announce("batched silu+quant bf16 weight, 300 experts")
+    counts = zipf_counts(6000, 300, seed=5, n_empty=7)
+    _batched_case(gpu, counts, 512, 1.0, 1.0, seed=34, wdtype=torch.bfloat16)
