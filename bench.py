@@ -1,0 +1,367 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused blockwise-FP8 quantisation path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs all|cfg1,cfg2,...] [--no-cpu]
+
+A "step" is one call of the entry point of a configuration on one batch of
+synthetic (seeded) input that is already resident in HBM.  Calls go through
+the C ABI with preallocated outputs; K steps are timed between two events on
+the launch stream.  Buffers rotate over enough copies to exceed twice the
+256 MB Infinity Cache, so the figure is an HBM figure ("cold"); the same loop
+on one fixed set of buffers gives the cache-resident ("hot") figure.
+
+Prints ONE JSON line: the headline metric is us/call of RMSNorm + 1x128 quant
+forward on bf16 [8192, 2048] (output_mode 2); the other configurations are
+listed under "configs".
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+INFINITY_CACHE_BYTES = 256 << 20
+FP8 = torch.float8_e4m3fn
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+class Case:
+    """One configuration: `sets` buffer sets and a launcher taking a set index."""
+
+    def __init__(self, name, entry, shape, algo_bytes, make_set, launch, cpu_fn):
+        self.name, self.entry, self.shape = name, entry, shape
+        self.algo_bytes = algo_bytes
+        self.make_set, self.launch, self.cpu_fn = make_set, launch, cpu_fn
+        self.sets = []
+
+    def allocate(self):
+        n_sets = max(2, min(16, (2 * INFINITY_CACHE_BYTES + 64 * (1 << 20)) // max(1, self.algo_bytes) + 1))
+        self.sets = [self.make_set() for _ in range(n_sets)]
+
+
+def build_cases(names, dev):
+    from linghe_amd import _lib, configs
+    L = _lib.lib
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    cases = {}
+
+    def add(name, **kw):
+        if names is None or name in names:
+            cases[name] = kw
+
+    # ---------------------------------------------------------------- cfg1 / cfg5b / cfg5c
+    def rms_quant_case(name, data, mode):
+        x_cpu, g_cpu, eps = data["x"], data["gamma"], data["eps"]
+        M, n = x_cpu.shape
+        gd = g_cpu.to(dev)
+        rstd_saved = None
+        if mode == 1:
+            from linghe_amd.utils.norm import triton_rms_norm_forward
+            _, rstd_saved = triton_rms_norm_forward(x_cpu.to(dev), gd, eps)
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev))
+            if mode != 1:
+                s["q"] = torch.empty((M, n), device=dev, dtype=FP8)
+                s["s"] = torch.empty((n // 128, M), device=dev, dtype=torch.float32)
+                s["rstd"] = torch.empty((M,), device=dev, dtype=torch.float32)
+            else:
+                s["q"], s["s"], s["rstd"] = None, None, rstd_saved.clone()
+            if mode != 0:
+                s["qt"] = torch.empty((n, M), device=dev, dtype=FP8)
+                s["st"] = torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32)
+            else:
+                s["qt"], s["st"] = None, None
+            s["args"] = (_p(s["x"]), _p(gd), _p(s["q"]), _p(s["s"]), _p(s["rstd"]), _p(s["qt"]), _p(s["st"]),
+                         M, n, float(eps), 0, mode, _lib.FQ_E4M3, stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_rmsnorm_quant_fwd(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.rms_norm_and_block_quant_forward(x_cpu, g_cpu, eps, False)
+
+        return Case(name, "triton_rms_norm_and_block_quant_forward(output_mode=%d)" % mode, [M, n],
+                    configs.bytes_rmsnorm_quant(M, n, mode), make_set, launch, cpu_fn)
+
+    lazy = {}
+
+    def cfg5():
+        if "cfg5" not in lazy:
+            lazy["cfg5"] = configs.cfg5_rmsnorm_large()
+        return lazy["cfg5"]
+
+    add("cfg1", build=lambda: rms_quant_case("cfg1", configs.cfg1_rmsnorm_quant(), 2))
+    add("cfg5b", build=lambda: rms_quant_case("cfg5b", cfg5(), 2))
+    add("cfg5c", build=lambda: rms_quant_case("cfg5c", cfg5(), 1))
+
+    # ---------------------------------------------------------------- cfg2
+    def swiglu_fwd_case():
+        x_cpu = configs.cfg2_swiglu_fwd()["x"]
+        M, N = x_cpu.shape
+        n = N // 2
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), q=torch.empty((M, n), device=dev, dtype=FP8),
+                     s=torch.empty((n // 128, M), device=dev, dtype=torch.float32),
+                     qt=torch.empty((n, M), device=dev, dtype=FP8),
+                     st=torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32))
+            s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, 0, 2,
+                         _lib.FQ_E4M3, stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_swiglu_quant_fwd(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.silu_and_block_quant_forward(x_cpu, False)
+
+        return Case("cfg2", "triton_silu_and_block_quant_forward(output_mode=2)", [M, N],
+                    configs.bytes_swiglu_fwd(M, n), make_set, launch, cpu_fn)
+
+    add("cfg2", build=swiglu_fwd_case)
+
+    # ---------------------------------------------------------------- cfg3 (+ backward)
+    def batched_case(backward):
+        d = lazy.setdefault("cfg3", configs.cfg3_batched_swiglu())
+        x_cpu, w_cpu, counts, dy_cpu = d["x"], d["weight"], d["counts"], d["dy"]
+        M, N = x_cpu.shape
+        n = N // 2
+        E = len(counts)
+        blocks = sum((c + 127) // 128 for c in counts)
+        cnt = torch.tensor(counts, dtype=torch.int32, device=dev)
+        W = N if backward else n
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), w=w_cpu.to(dev), q=torch.empty((M, W), device=dev, dtype=FP8),
+                     s=torch.empty((M, W // 128), device=dev, dtype=torch.float32),
+                     qt=torch.empty((M, W), device=dev, dtype=FP8),
+                     st=torch.empty((blocks, W), device=dev, dtype=torch.float32))
+            if backward:
+                s["dy"] = dy_cpu.to(dev)
+                s["dw"] = torch.empty((M, 1), device=dev, dtype=torch.float32)
+                s["dws"] = torch.empty((M, n // 128), device=dev, dtype=torch.float32)
+                s["args"] = (_p(s["dy"]), _p(s["x"]), _p(s["w"]), 0, _p(cnt), 0, E, blocks, _p(s["q"]), _p(s["s"]),
+                             _p(s["dw"]), _p(s["qt"]), _p(s["st"]), _p(s["dws"]), M, n, 0, _lib.FQ_E4M3, stream)
+            else:
+                s["args"] = (_p(s["x"]), _p(s["w"]), 0, _p(cnt), 0, E, blocks, _p(s["q"]), _p(s["s"]), _p(s["qt"]),
+                             _p(s["st"]), M, n, 0, 2, _lib.FQ_E4M3, stream)
+            return s
+
+        if backward:
+            def launch(s):
+                _lib.check(L.fq_batched_swiglu_quant_bwd(*s["args"]))
+
+            def cpu_fn():
+                from oracle import fq_oracle as O
+                return O.batch_weighted_silu_and_block_quant_backward(dy_cpu, x_cpu, w_cpu, counts, False)
+            nbytes = configs.bytes_batched_swiglu_bwd(M, n, counts)
+            entry = "triton_batch_weighted_silu_and_block_quant_backward"
+        else:
+            def launch(s):
+                _lib.check(L.fq_batched_swiglu_quant_fwd(*s["args"]))
+
+            def cpu_fn():
+                from oracle import fq_oracle as O
+                return O.batch_weighted_silu_and_block_quant_forward(x_cpu, w_cpu, counts, False)
+            nbytes = configs.bytes_batched_swiglu_fwd(M, n, counts)
+            entry = "triton_batch_weighted_silu_and_block_quant_forward(output_mode=2)"
+        c = Case("cfg3b" if backward else "cfg3", entry, [M, N], nbytes, make_set, launch, cpu_fn)
+        c.extra = dict(n_experts=E, blocks=blocks, empty_experts=sum(1 for v in counts if v == 0),
+                       max_count=max(counts))
+        return c
+
+    add("cfg3", build=lambda: batched_case(False))
+    add("cfg3b", build=lambda: batched_case(True))
+
+    # ---------------------------------------------------------------- cfg4
+    def swiglu_bwd_case(kind, name):
+        d = lazy.setdefault("cfg4", configs.cfg4_swiglu_bwd())
+        dy_cpu, x_cpu = d["dy"], d["x"]
+        M, N = x_cpu.shape
+        n = N // 2
+        dt = FP8 if kind == _lib.FQ_E4M3 else torch.float8_e5m2
+
+        def make_set():
+            s = dict(dy=dy_cpu.to(dev), x=x_cpu.to(dev), q=torch.empty((M, N), device=dev, dtype=dt),
+                     s=torch.empty((N // 128, M), device=dev, dtype=torch.float32),
+                     qt=torch.empty((N, M), device=dev, dtype=dt),
+                     st=torch.empty((M // 128, N), device=dev, dtype=torch.float32))
+            s["args"] = (_p(s["dy"]), _p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, 0, kind,
+                         stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_swiglu_quant_bwd(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.silu_and_block_quant_backward(dy_cpu, x_cpu, False, dt)
+
+        return Case(name, "triton_silu_and_block_quant_backward(fp8=%s)" % str(dt).split(".")[-1], [M, N],
+                    configs.bytes_swiglu_bwd(M, n), make_set, launch, cpu_fn)
+
+    add("cfg4", build=lambda: swiglu_bwd_case(_lib.FQ_E4M3, "cfg4"))
+    add("cfg4_e5m2", build=lambda: swiglu_bwd_case(_lib.FQ_E5M2, "cfg4_e5m2"))
+
+    # ---------------------------------------------------------------- cfg5a
+    def rms_bwd_case():
+        d = cfg5()
+        x_cpu, g_cpu, dy_cpu, eps = d["x"], d["gamma"], d["dy"], d["eps"]
+        M, n = x_cpu.shape
+        gd = g_cpu.to(dev)
+        n_part = int(L.fq_rmsnorm_bwd_num_partials(M, n))
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), dy=dy_cpu.to(dev), dx=torch.empty((M, n), device=dev, dtype=torch.bfloat16),
+                     dg=torch.empty((n,), device=dev, dtype=torch.float32),
+                     part=torch.empty((n_part, n), device=dev, dtype=torch.float32))
+            s["args"] = (_p(s["dy"]), _p(s["x"]), _p(gd), None, _p(s["dx"]), _p(s["dg"]), _p(s["part"]), n_part, M, n,
+                         float(eps), stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_rmsnorm_bwd(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.rms_norm_backward(x_cpu, g_cpu, dy_cpu, eps)
+
+        return Case("cfg5a", "triton_rms_norm_backward", [M, n], configs.bytes_rmsnorm_bwd(M, n), make_set, launch,
+                    cpu_fn)
+
+    add("cfg5a", build=rms_bwd_case)
+    return cases
+
+
+def time_loop(case, sets, steps, warmup):
+    """us per call: `steps` back-to-back launches between two events on the
+    launch stream (the current torch stream), rotating over `sets`."""
+    k = len(sets)
+    for i in range(warmup):
+        case.launch(sets[i % k])
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        case.launch(sets[i % k])
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) * 1000.0 / steps
+
+
+def time_cpu(case, budget_s):
+    """oracle on the host cores: 1 warm-up, then min over up to 3 runs within the budget."""
+    t0 = time.perf_counter()
+    case.cpu_fn()
+    first = time.perf_counter() - t0
+    runs = [first]
+    spent = first
+    while len(runs) < 4 and spent + runs[-1] < budget_s:
+        t0 = time.perf_counter()
+        case.cpu_fn()
+        runs.append(time.perf_counter() - t0)
+        spent += runs[-1]
+    best = min(runs[1:]) if len(runs) > 1 else runs[0]
+    return best * 1e6, len(runs)
+
+
+ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c"]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--configs", default="all")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--cpu-all", action="store_true", help="time the CPU oracle for every config, not only cfg1")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU (every row block / expert is independent, "
+              "there is no collective to time); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    names = ALL if args.configs == "all" else [c.strip() for c in args.configs.split(",")]
+    if "cfg1" not in names:
+        names = ["cfg1"] + names
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    builders = build_cases(set(names), dev)
+    results = {}
+    headline_cpu = None
+    for name in names:
+        case = builders[name]["build"]()
+        case.allocate()
+        cold = time_loop(case, case.sets, args.steps, args.warmup)
+        hot = time_loop(case, case.sets[:1], args.steps, args.warmup)
+        gbs = case.algo_bytes / cold / 1e3
+        r = dict(entry=case.entry, shape=case.shape, algorithmic_bytes=case.algo_bytes,
+                 us_per_call=round(cold, 3), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
+                 us_per_call_hot=round(hot, 3), gb_per_s_hot=round(case.algo_bytes / hot / 1e3, 1),
+                 buffer_sets=len(case.sets))
+        if hasattr(case, "extra"):
+            r.update(case.extra)
+        if not args.no_cpu and (name == "cfg1" or args.cpu_all):
+            cpu_us, n_runs = time_cpu(case, budget_s=20.0)
+            r["cpu_us_per_call"] = round(cpu_us, 1)
+            r["cpu_runs"] = n_runs
+            if name == "cfg1":
+                headline_cpu = (cpu_us, n_runs)
+        results[name] = r
+        print(f"[bench] {name}: {cold:.2f} us cold ({gbs:.0f} GB/s, {100 * gbs / HBM_PEAK_GBS:.1f}% of peak), "
+              f"{hot:.2f} us hot", file=sys.stderr, flush=True)
+        case.sets = []
+        del case
+        torch.cuda.empty_cache()
+
+    head = results["cfg1"]
+    line = {
+        "metric": "us/call and achieved HBM GB/s (% of peak), RMSNorm+quant fwd 8192x2048",
+        "value": head["us_per_call"],
+        "unit": "us/call",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["us_per_call"] / 1000.0, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cfg1: RMSNorm + 1x128/128x1 e4m3 blockwise quant forward, x bf16 [8192,2048], "
+                               "output_mode 2, round_scale False, buffers rotated beyond the Infinity Cache",
+                   "entry": head["entry"]},
+        "roofline": {"bound": "hbm", "achieved": head["gb_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["frac_of_hbm_peak"], "traffic": None},
+        "configs": results,
+    }
+    if headline_cpu is not None:
+        line["cpu_baseline"] = {"value": round(headline_cpu[0], 1), "unit": "us/call",
+                                "cores": torch.get_num_threads(), "kind": "port",
+                                "sample": "cfg1 at full size, torch CPU oracle, 1 warm-up + min of %d calls; "
+                                          "os.cpu_count()=%d" % (max(1, headline_cpu[1] - 1), os.cpu_count())}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

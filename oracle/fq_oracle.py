@@ -136,10 +136,18 @@ def rms_norm_backward_closed_form(x, weight, dy, eps: float = 1e-6):
 
 
 def rms_norm_and_block_quant_forward(x, weight, eps: float = 1e-6,
-                                     round_scale: bool = False, fp8_dtype=E4M3):
+                                     round_scale: bool = False, fp8_dtype=E4M3, rstd=None):
     """tests/test_norm.py:70-84.  Returns q [M,n], scale [n/128,M], rstd [M],
-    qt [n,M], tscale [ceil(M/128), n]."""
-    y, rstd = rms_norm_fp32(x, weight, eps)
+    qt [n,M], tscale [ceil(M/128), n].
+
+    With ``rstd`` given, the normalised value is (x * rstd[row]) * weight, the
+    expression the reference evaluates when the caller passes a saved statistic
+    (linghe/utils/norm.py:331-333, output_mode 1)."""
+    if rstd is None:
+        y, rstd = rms_norm_fp32(x, weight, eps)
+    else:
+        rstd = rstd.float()
+        y = (x.float() * rstd.reshape(-1, 1)) * weight.float()
     q, s, qt, st = blockwise_quant(y, round_scale, fp8_dtype)
     return q, s, rstd, qt, st
 
