@@ -246,6 +246,23 @@ def build_cases(names, dev):
                     cpu_fn)
 
     add("cfg5a", build=rms_bwd_case)
+
+    # ---------------------------------------------------------------- plain copy of known size
+    # (calibration of the FETCH_SIZE / WRITE_SIZE counters: reads and writes 256 MiB)
+    def copy_case():
+        nbytes = 256 << 20
+
+        def make_set():
+            return dict(src=torch.zeros(nbytes // 2, device=dev, dtype=torch.bfloat16),
+                        dst=torch.empty(nbytes // 2, device=dev, dtype=torch.bfloat16))
+
+        def launch(s):
+            s["dst"].copy_(s["src"])
+
+        return Case("copy", "torch copy_ of 256 MiB (counter calibration)", [nbytes], 2 * nbytes, make_set, launch,
+                    lambda: None)
+
+    add("copy", build=copy_case)
     return cases
 
 
@@ -293,6 +310,9 @@ def main():
     ap.add_argument("--configs", default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--cpu-all", action="store_true", help="time the CPU oracle for every config, not only cfg1")
+    ap.add_argument("--no-headline", action="store_true",
+                    help="profiling aid: run only the named configs and print their results without the headline line")
+    ap.add_argument("--hot-only", action="store_true", help="profiling aid: one buffer set, no rotation")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (every row block / expert is independent, "
@@ -302,7 +322,7 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     names = ALL if args.configs == "all" else [c.strip() for c in args.configs.split(",")]
-    if "cfg1" not in names:
+    if "cfg1" not in names and not args.no_headline:
         names = ["cfg1"] + names
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -312,8 +332,10 @@ def main():
     for name in names:
         case = builders[name]["build"]()
         case.allocate()
+        if args.hot_only:
+            case.sets = case.sets[:1]
         cold = time_loop(case, case.sets, args.steps, args.warmup)
-        hot = time_loop(case, case.sets[:1], args.steps, args.warmup)
+        hot = cold if args.hot_only else time_loop(case, case.sets[:1], args.steps, args.warmup)
         gbs = case.algo_bytes / cold / 1e3
         r = dict(entry=case.entry, shape=case.shape, algorithmic_bytes=case.algo_bytes,
                  us_per_call=round(cold, 3), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
@@ -334,6 +356,9 @@ def main():
         del case
         torch.cuda.empty_cache()
 
+    if args.no_headline:
+        print(json.dumps({"configs": results}))
+        return
     head = results["cfg1"]
     line = {
         "metric": "us/call and achieved HBM GB/s (% of peak), RMSNorm+quant fwd 8192x2048",

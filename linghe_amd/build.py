@@ -26,6 +26,10 @@ HIPCC_FLAGS = [
     "-fPIC",
     # parity with the fp32 CPU oracle needs separate mul/add roundings
     "-ffp-contract=off",
+    # NaNs are not part of the contract of these kernels: lets fmaxf be a single
+    # v_max_f32 (no canonicalisation) and DPP moves fold into their consumer
+    "-fno-honor-nans",
+    "-mno-amdgpu-ieee",
     # packed fp32 VALU ops are not to be generated for this machine pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",

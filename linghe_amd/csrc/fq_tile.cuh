@@ -88,9 +88,11 @@ __device__ __forceinline__ void store_t_chunk(uint8_t* dst, const uint4& v, int 
 
 // Quantise the tile held in registers (v[s][j] = element (rg*RPT+s, cg*8+j);
 // rows >= rows_valid must hold 0).  All threads of the workgroup must call it.
-template <int KIND, bool ROUND, int MODE, int RPT, bool EXACT_DIV = true>
-__device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o,
-                                              TileShared<RPT>& sh) {
+// FULL: the tile has all 128 rows and its transposed rows are 16-byte aligned,
+// so no store needs a mask.
+template <int KIND, bool ROUND, int MODE, int RPT, bool FULL, bool EXACT_DIV = true>
+__device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], const TileOut& o,
+                                                   TileShared<RPT>& sh) {
   using Shape = TileShape<RPT>;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -117,13 +119,13 @@ __device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const Ti
       pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
       pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
       const int i = rg * RPT + s;
-      if (i < o.rows_valid) *(uint2*)(o.q + o.q_off + (int64_t)i * o.q_ld + cg * 8) = pk;
+      if (FULL || i < o.rows_valid) *(uint2*)(o.q + o.q_off + (int64_t)i * o.q_ld + cg * 8) = pk;
     }
     // lane cg < RPT of each row group stores the scale of row rg*RPT+cg:
     // a wave writes 4*RPT consecutive floats
     if (cg < RPT) {
       const int i = rg * RPT + cg;
-      if (i < o.rows_valid) o.s[o.s_off + i] = my_scale;
+      if (FULL || i < o.rows_valid) o.s[o.s_off + i] = my_scale;
     }
   }
 
@@ -187,10 +189,22 @@ __device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const Ti
     for (int k = 0; k < kGroup / kRowsPerPass; ++k) {
       const int c = (tid >> 3) + k * kRowsPerPass;
       const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
-      store_t_chunk(o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16, val, o.rows_valid - ch * 16);
+      uint8_t* dst = o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16;
+      if constexpr (FULL) *(uint4*)dst = val;
+      else store_t_chunk(dst, val, o.rows_valid - ch * 16);
     }
     __syncthreads();  // LDS is reused by a following call
   }
+}
+
+template <int KIND, bool ROUND, int MODE, int RPT, bool EXACT_DIV = true>
+__device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o,
+                                              TileShared<RPT>& sh) {
+  // workgroup-uniform choice of the mask-free path
+  bool full = o.rows_valid == kGroup;
+  if constexpr (MODE != 0) full = full && ((((uintptr_t)(o.qt + o.t_off)) | (uintptr_t)o.t_ld) & 15) == 0;
+  if (full) quantize_tile_impl<KIND, ROUND, MODE, RPT, true, EXACT_DIV>(v, o, sh);
+  else quantize_tile_impl<KIND, ROUND, MODE, RPT, false, EXACT_DIV>(v, o, sh);
 }
 
 // ---------------------------------------------------------------------------

@@ -92,11 +92,16 @@ template <int RPT>
 __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
+  const uint16_t* p = base + (int64_t)(rg * RPT) * ld + cg * 8;
+  if (rows_valid == kGroup) {  // workgroup-uniform: no per-row masks
 #pragma unroll
-  for (int s = 0; s < RPT; ++s) {
-    const int i = rg * RPT + s;
-    raw[s] = make_uint4(0, 0, 0, 0);
-    if (i < rows_valid) raw[s] = *(const uint4*)(base + (int64_t)i * ld + cg * 8);
+    for (int s = 0; s < RPT; ++s) raw[s] = *(const uint4*)(p + (int64_t)s * ld);
+  } else {
+#pragma unroll
+    for (int s = 0; s < RPT; ++s) {
+      raw[s] = make_uint4(0, 0, 0, 0);
+      if (rg * RPT + s < rows_valid) raw[s] = *(const uint4*)(p + (int64_t)s * ld);
+    }
   }
 }
 
