@@ -29,6 +29,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+TWO_PASS = False  # --two-pass: RMSNorm+quant mode 2 without the workspace (statistic kernel + tile kernel)
 INFINITY_CACHE_BYTES = 256 << 20
 FP8 = torch.float8_e4m3fn
 
@@ -84,8 +85,9 @@ def build_cases(names, dev):
                 s["st"] = torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32)
             else:
                 s["qt"], s["st"] = None, None
+            ws, ws_bytes = _lib.norm_workspace(s["x"], M, n) if (mode == 2 and not TWO_PASS) else (None, 0)
             s["args"] = (_p(s["x"]), _p(gd), _p(s["q"]), _p(s["s"]), _p(s["rstd"]), _p(s["qt"]), _p(s["st"]),
-                         M, n, float(eps), 0, mode, _lib.FQ_E4M3, stream)
+                         M, n, float(eps), 0, mode, _lib.FQ_E4M3, _p(ws), ws_bytes, stream)
             return s
 
         def launch(s):
@@ -313,6 +315,8 @@ def main():
     ap.add_argument("--no-headline", action="store_true",
                     help="profiling aid: run only the named configs and print their results without the headline line")
     ap.add_argument("--hot-only", action="store_true", help="profiling aid: one buffer set, no rotation")
+    ap.add_argument("--two-pass", action="store_true",
+                    help="run RMSNorm+quant mode 2 as statistic kernel + tile kernel (no workspace)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (every row block / expert is independent, "
@@ -321,6 +325,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    global TWO_PASS
+    TWO_PASS = args.two_pass
     names = ALL if args.configs == "all" else [c.strip() for c in args.configs.split(",")]
     if "cfg1" not in names and not args.no_headline:
         names = ["cfg1"] + names

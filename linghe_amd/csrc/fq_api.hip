@@ -5,6 +5,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "fq_launch.h"
 
 namespace {
@@ -148,9 +150,26 @@ int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float
                       fn);
 }
 
+int64_t fq_rmsnorm_quant_workspace_bytes(int64_t M, int64_t n) {
+  if (M <= 0 || n <= 0 || n % 128 != 0 || n > 8192) return 0;
+  return fq::rmsnorm_fused_scratch_bytes(M, (int)n);
+}
+
+// stamp of the next single-pass launch (never 0: a cleared workspace reads as "not ready")
+static std::atomic<uint32_t> g_stamp{0};
+static uint32_t next_stamp() {
+  uint32_t t;
+  do { t = g_stamp.fetch_add(1u) + 1u; } while (t == 0u);
+  return t;
+}
+
+static std::atomic<int> g_wait_limit{0};
+
+void fq_set_wait_limit(int polls) { g_wait_limit.store(polls > 0 ? polls : 0); }
+
 int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt, float* st,
                          int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
-                         void* stream) {
+                         void* workspace, int64_t workspace_bytes, void* stream) {
   const char* fn = "fq_rmsnorm_quant_fwd";
   int rc = check_common(fn, M, n, round_scale, fp8_kind);
   if (rc) return rc;
@@ -160,18 +179,42 @@ int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, fl
   FQ_REQUIRE(x && gamma && rstd, FQ_ERR_ARG, "%s: NULL pointer", fn);
   FQ_REQUIRE(aligned16(x) && aligned16(gamma), FQ_ERR_ARG, "%s: misaligned pointer", fn);
   hipStream_t st_ = (hipStream_t)stream;
-  if (output_mode == 0 || output_mode == 2) {
-    rc = check_launch(fq::launch_rmsnorm_fwd(x, gamma, q, s, rstd, M, (int)n, eps, 0, 1, round_scale, fp8_kind, st_),
+  if ((rc = check_tiles(fn, ((M + 127) / 128) * (n / 128)))) return rc;
+  // The single-pass kernel keeps every tile in registers while its slab's statistic
+  // is assembled; that pays only while the whole grid is resident at once (4
+  // workgroups on each of the 256 CUs).  Larger problems run as two passes.
+  bool single_pass = output_mode == 2 && workspace != nullptr && ((M + 127) / 128) * (n / 128) <= 1024;
+  if (single_pass) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st_, &cap) != hipSuccess) {
+      (void)hipGetLastError();
+      cap = hipStreamCaptureStatusNone;
+    }
+    if (cap != hipStreamCaptureStatusNone) single_pass = false;  // a replay would reuse the stamp
+  }
+  if (single_pass) {
+    FQ_REQUIRE(workspace_bytes >= fq::rmsnorm_fused_scratch_bytes(M, (int)n), FQ_ERR_ARG,
+               "%s: workspace of %lld bytes is smaller than fq_rmsnorm_quant_workspace_bytes", fn,
+               (long long)workspace_bytes);
+    FQ_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FQ_ERR_ARG,
+               "%s: workspace must be 256-byte aligned", fn);
+    return check_launch(fq::launch_rmsnorm_quant_fused(x, gamma, q, s, rstd, qt, st, workspace, next_stamp(), M,
+                                                       (int)n, eps, round_scale, 2, fp8_kind, g_wait_limit.load(),
+                                                       st_),
+                        fn);
+  }
+  if (output_mode == 0) {
+    return check_launch(fq::launch_rmsnorm_fwd(x, gamma, q, s, rstd, M, (int)n, eps, 0, 1, round_scale, fp8_kind, st_),
+                        fn);
+  }
+  if (output_mode == 2) {  // two passes: the statistic alone, then the tile kernel with both outputs
+    rc = check_launch(fq::launch_rmsnorm_fwd(x, gamma, nullptr, nullptr, rstd, M, (int)n, eps, 0, 2, 0, FQ_E4M3, st_),
                       fn);
     if (rc) return rc;
   }
-  if (output_mode == 1 || output_mode == 2) {
-    if ((rc = check_tiles(fn, ((M + 127) / 128) * (n / 128)))) return rc;
-    rc = check_launch(fq::launch_rmsnorm_quant_tile(x, gamma, rstd, nullptr, nullptr, qt, st, M, (int)n, round_scale,
-                                                    1, fp8_kind, st_),
+  return check_launch(fq::launch_rmsnorm_quant_tile(x, gamma, rstd, q, s, qt, st, M, (int)n, round_scale, output_mode,
+                                                    fp8_kind, st_),
                       fn);
-  }
-  return rc;
 }
 
 int fq_swiglu_quant_fwd(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t n,

@@ -51,6 +51,17 @@ __device__ __forceinline__ uint4 pack8_bf16(const float (&v)[8]) {
   return o;
 }
 
+// sum of squares of 8 packed bf16 with the bf16 dot-product instruction: the
+// products are exact in fp32, the additions round in a fixed order
+__device__ __forceinline__ float sumsq8(const uint4& p) {
+  float ss = 0.f;
+  ss = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p.x), __builtin_bit_cast(bf16x2_t, p.x), ss, false);
+  ss = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p.y), __builtin_bit_cast(bf16x2_t, p.y), ss, false);
+  ss = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p.z), __builtin_bit_cast(bf16x2_t, p.z), ss, false);
+  ss = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p.w), __builtin_bit_cast(bf16x2_t, p.w), ss, false);
+  return ss;
+}
+
 // 4 fp32 -> 4 fp8 codes in one dword (native converts, RNE)
 template <int KIND>
 __device__ __forceinline__ uint32_t pack4_fp8(float a, float b, float c, float d) {

@@ -63,19 +63,14 @@ template <int NCHUNK>
 __device__ __forceinline__ float sumsq(const uint4 (&raw)[NCHUNK]) {
   float ss = 0.f;
 #pragma unroll
-  for (int k = 0; k < NCHUNK; ++k) {
-    float a[8];
-    unpack8(raw[k], a);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(a[j], a[j], ss);
-  }
+  for (int k = 0; k < NCHUNK; ++k) ss += sumsq8(raw[k]);
   return ss;
 }
 
 // ---------------------------------------------------------------------------
-// forward: OUT_QUANT=false -> bf16 y ; OUT_QUANT=true -> fp8 codes + [nb, M] scales
+// forward: OUT = 0 -> bf16 y ; 1 -> fp8 codes + [nb, M] scales ; 2 -> rstd only
 // ---------------------------------------------------------------------------
-template <int T, int NCHUNK, bool REUSE, bool OUT_QUANT, int KIND, bool ROUND>
+template <int T, int NCHUNK, bool REUSE, int OUT, int KIND, bool ROUND>
 __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restrict__ x,
                                                         const uint16_t* __restrict__ gamma, void* __restrict__ out,
                                                         float* __restrict__ scale, float* __restrict__ rstd,
@@ -83,7 +78,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
   __shared__ RowShared<T> sh;
   const int tid = threadIdx.x;
   uint4 gm[NCHUNK];
-  load_row<T, NCHUNK>(gamma, n, gm);
+  if constexpr (OUT != 2) load_row<T, NCHUNK>(gamma, n, gm);
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
   int64_t r1 = r0 + rows_per_wg;
   if (r1 > M) r1 = M;
@@ -99,6 +94,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
       r = rstd_from_sumsq(ss, n, eps);
       if (tid == 0) rstd[row] = r;
     }
+    if constexpr (OUT == 2) return;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
       const int c = tid + k * T;
@@ -107,7 +103,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
       unpack8(gm[k], w);
 #pragma unroll
       for (int j = 0; j < 8; ++j) y[j] = (a[j] * r) * w[j];
-      if constexpr (!OUT_QUANT) {
+      if constexpr (OUT == 0) {
         if (c * 8 < n) *(uint4*)((uint16_t*)out + row * n + c * 8) = pack8_bf16(y);
       } else {
         float m = 0.f;
@@ -167,7 +163,9 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
   if (r1 > M) r1 = M;
 
   auto process = [&](const uint4 (&rx)[NCHUNK], const uint4 (&rg)[NCHUNK], int64_t row, int parity) {
-    float ss = 0.f, dot = 0.f;
+    // the sum of squares is taken exactly as the forward kernels take it, so that a
+    // recomputed statistic equals a saved one bit for bit
+    float ss = REUSE ? 0.f : sumsq<NCHUNK>(rx), dot = 0.f;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
       float a[8], g[8], w[8];
@@ -175,10 +173,7 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
       unpack8(rg[k], g);
       unpack8(gm[k], w);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        ss = __builtin_fmaf(a[j], a[j], ss);
-        dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
-      }
+      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
     }
     block_sum2<T>(ss, dot, sh, parity);
     float r;
@@ -317,12 +312,15 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
   FQ_ROW_SHAPES(hipLaunchKernelGGL((rmsnorm_fwd_kernel<kT, kNC, REUSE, QUANT, KINDV, ROUNDV>), grid,       \
                                    dim3(kT), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, out,   \
                                    scale, rstd, M, n, eps, rows_per_wg);)
-  if (!quant) {
-    if (reuse_rstd) { FQ_LAUNCH_FWD(true, false, kE4M3, false) } else { FQ_LAUNCH_FWD(false, false, kE4M3, false) }
+  // quant: 0 = bf16 output, 1 = fp8 codes + scales, 2 = statistic only
+  if (quant == 2) {
+    FQ_LAUNCH_FWD(false, 2, kE4M3, false)
+  } else if (!quant) {
+    if (reuse_rstd) { FQ_LAUNCH_FWD(true, 0, kE4M3, false) } else { FQ_LAUNCH_FWD(false, 0, kE4M3, false) }
   } else if (kind == kE5M2) {
-    if (round_scale) { FQ_LAUNCH_FWD(false, true, kE5M2, true) } else { FQ_LAUNCH_FWD(false, true, kE5M2, false) }
+    if (round_scale) { FQ_LAUNCH_FWD(false, 1, kE5M2, true) } else { FQ_LAUNCH_FWD(false, 1, kE5M2, false) }
   } else {
-    if (round_scale) { FQ_LAUNCH_FWD(false, true, kE4M3, true) } else { FQ_LAUNCH_FWD(false, true, kE4M3, false) }
+    if (round_scale) { FQ_LAUNCH_FWD(false, 1, kE4M3, true) } else { FQ_LAUNCH_FWD(false, 1, kE4M3, false) }
   }
 #undef FQ_LAUNCH_FWD
   return hipGetLastError();

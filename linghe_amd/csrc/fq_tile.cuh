@@ -44,7 +44,8 @@ template <int RPT>
 struct alignas(16) TileShared {
   uint8_t t[kGroup * kGroup];                       // transposed codes, 16-byte chunks XOR-swizzled
   float colmax[TileShape<RPT>::kWaves][kGroup];      // per-wave column amax
-  float cscale[kGroup];                              // column scales
+  float2 cdiv[kGroup];                               // per column {scale, 1/scale}
+  float2 rdiv[kGroup];                               // per row    {scale, 1/scale}
 };
 
 // xor-16 / xor-32 lane exchange + max with the gfx950 permlane swaps
@@ -102,16 +103,35 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
 
   // ------------------------------------------------------------- row-wise
   if constexpr (MODE == 0 || MODE == 2) {
-    float my_scale = 0.f;
+    // every lane of a 16-lane row gets the amax of its RPT rows; lane cg < RPT then
+    // turns ONE of them (row rg*RPT+cg) into {scale, 1/scale}, stores the scale,
+    // and hands the pair to the other lanes through LDS.  The rows of a wave are
+    // written and read by that wave only, so no barrier is needed.
+    float mine = 0.f;
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
       float m = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[s][j]));
       m = row16_max(m);
-      const float sc = make_scale<KIND, ROUND>(m);
-      if (cg == s) my_scale = sc;
+      if (cg == s) mine = m;
+    }
+    if (cg < RPT) {
+      const float sc = make_scale<KIND, ROUND>(mine);
       const Divisor d = make_divisor(sc);
+      const int i = rg * RPT + cg;
+      sh.rdiv[i] = make_float2(d.s, d.r);
+      if (FULL || i < o.rows_valid) o.s[o.s_off + i] = sc;  // a wave writes 4*RPT consecutive floats
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int s = 0; s < RPT; ++s) {
+      const float2 sr = sh.rdiv[rg * RPT + s];
+      Divisor d;
+      d.s = sr.x;
+      d.r = sr.y;
       float qv[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) qv[j] = EXACT_DIV ? div_exact(v[s][j], d) : v[s][j] * d.r;
@@ -120,12 +140,6 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
       const int i = rg * RPT + s;
       if (FULL || i < o.rows_valid) *(uint2*)(o.q + o.q_off + (int64_t)i * o.q_ld + cg * 8) = pk;
-    }
-    // lane cg < RPT of each row group stores the scale of row rg*RPT+cg:
-    // a wave writes 4*RPT consecutive floats
-    if (cg < RPT) {
-      const int i = rg * RPT + cg;
-      if (FULL || i < o.rows_valid) o.s[o.s_off + i] = my_scale;
     }
   }
 
@@ -150,16 +164,20 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
 #pragma unroll
       for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[w][tid]);
       const float sc = make_scale<KIND, ROUND>(m);
-      sh.cscale[tid] = sc;
+      const Divisor d = make_divisor(sc);
+      sh.cdiv[tid] = make_float2(d.s, d.r);
       o.st[o.st_off + tid] = sc;
     }
     __syncthreads();
-    float cs[8];
+    Divisor cd[8];
     {
-      const float4* src = (const float4*)&sh.cscale[cg * 8];
-      const float4 a = src[0], b = src[1];
-      cs[0] = a.x; cs[1] = a.y; cs[2] = a.z; cs[3] = a.w;
-      cs[4] = b.x; cs[5] = b.y; cs[6] = b.z; cs[7] = b.w;
+      const float4* src = (const float4*)&sh.cdiv[cg * 8];
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const float4 a = src[h];
+        cd[2 * h].s = a.x; cd[2 * h].r = a.y;
+        cd[2 * h + 1].s = a.z; cd[2 * h + 1].r = a.w;
+      }
     }
     // transposed codes -> LDS; byte (c, i) lives at c*128 + ((i>>4) ^ ((c>>3)&7))*16 + (i&15)
     const int i0 = rg * RPT;
@@ -167,7 +185,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
     uint8_t* base = sh.t + chunk * 16 + (i0 & 15);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const Divisor d = make_divisor(cs[j]);
+      const Divisor d = cd[j];
       float qv[RPT];
 #pragma unroll
       for (int s = 0; s < RPT; ++s) qv[s] = EXACT_DIV ? div_exact(v[s][j], d) : v[s][j] * d.r;

@@ -1,0 +1,113 @@
+// Where a 128x128 tile of a launch lives: its rows, its column block and the
+// offsets of its four outputs, for the single-matrix and the per-expert forms.
+#pragma once
+#include "fq_tile.cuh"
+
+namespace fq {
+
+// ---------------------------------------------------------------------------
+// tile geometry
+// ---------------------------------------------------------------------------
+struct TileGeom {
+  int64_t row0;      // first global row of the tile
+  int rows_valid;
+  int cb;            // 128-column block of the input
+  int64_t s_base, s_stride;
+  int64_t t_base, t_stride;
+  int64_t st_row;
+  bool valid;
+};
+
+struct BatchArgs {
+  const void* counts;  // device, int32 or int64, [n_experts]
+  int counts_i64;
+  int n_experts;
+};
+
+// out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
+// backward's dx1|dx2)
+template <bool BATCHED, int THREADS>
+__device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out_w, const BatchArgs& b,
+                                                 ExpertScanShared& scan) {
+  TileGeom g;
+  const int id = blockIdx.x;
+  const int rbk = id / ncb;
+  g.cb = id - rbk * ncb;
+  if constexpr (!BATCHED) {
+    g.row0 = (int64_t)rbk * kGroup;
+    const int64_t left = M - g.row0;
+    g.rows_valid = left < kGroup ? (int)left : kGroup;
+    g.s_base = g.row0;
+    g.s_stride = M;
+    g.t_base = g.row0;
+    g.t_stride = M;
+    g.st_row = rbk;
+    g.valid = left > 0;
+  } else {
+    const ExpertTile et = find_expert_tile<THREADS>(b.counts, b.counts_i64, b.n_experts, rbk, scan);
+    g.valid = et.expert >= 0;
+    const int left = et.count - et.rb * kGroup;
+    g.rows_valid = left < kGroup ? left : kGroup;
+    g.row0 = et.row_start + (int64_t)et.rb * kGroup;
+    g.s_base = et.row_start * (out_w / kGroup) + (int64_t)et.rb * kGroup;
+    g.s_stride = et.count;
+    g.t_base = et.row_start * out_w + (int64_t)et.rb * kGroup;
+    g.t_stride = et.count;
+    g.st_row = et.tblock_start + et.rb;
+    if (g.row0 + g.rows_valid > M) g.valid = false;  // counts disagree with the matrix: write nothing
+  }
+  return g;
+}
+
+struct OutPtrs {
+  uint8_t* q;
+  float* s;
+  uint8_t* qt;
+  float* st;
+};
+
+// ocb: 128-column block index inside the quantised matrix of width out_w
+__device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g, int64_t out_w, int ocb) {
+  TileOut o;
+  o.q = p.q;
+  o.q_off = g.row0 * out_w + (int64_t)ocb * kGroup;
+  o.q_ld = out_w;
+  o.s = p.s;
+  o.s_off = g.s_base + (int64_t)ocb * g.s_stride;
+  o.qt = p.qt;
+  o.t_off = g.t_base + (int64_t)ocb * kGroup * g.t_stride;
+  o.t_ld = g.t_stride;
+  o.st = p.st;
+  o.st_off = g.st_row * out_w + (int64_t)ocb * kGroup;
+  o.rows_valid = g.rows_valid;
+  return o;
+}
+
+// RPT rows x 8 bf16 columns of a row-major matrix; rows >= rows_valid read as 0
+template <int RPT>
+__device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
+  const int cg = threadIdx.x & 15;
+  const int rg = threadIdx.x >> 4;
+  const uint16_t* p = base + (int64_t)(rg * RPT) * ld + cg * 8;
+  if (rows_valid == kGroup) {  // workgroup-uniform: no per-row masks
+#pragma unroll
+    for (int s = 0; s < RPT; ++s) raw[s] = *(const uint4*)(p + (int64_t)s * ld);
+  } else {
+#pragma unroll
+    for (int s = 0; s < RPT; ++s) {
+      raw[s] = make_uint4(0, 0, 0, 0);
+      if (rg * RPT + s < rows_valid) raw[s] = *(const uint4*)(p + (int64_t)s * ld);
+    }
+  }
+}
+
+#define FQ_DISPATCH_BOOL(flag, NAME, ...) \
+  if (flag) { constexpr bool NAME = true; __VA_ARGS__ } else { constexpr bool NAME = false; __VA_ARGS__ }
+#define FQ_DISPATCH_KIND(kind, NAME, ...) \
+  if ((kind) == kE5M2) { constexpr int NAME = kE5M2; __VA_ARGS__ } else { constexpr int NAME = kE4M3; __VA_ARGS__ }
+#define FQ_DISPATCH_MODE(mode, NAME, ...)                                    \
+  if ((mode) == 0) { constexpr int NAME = 0; __VA_ARGS__ }                   \
+  else if ((mode) == 1) { constexpr int NAME = 1; __VA_ARGS__ }              \
+  else { constexpr int NAME = 2; __VA_ARGS__ }
+
+}  // namespace fq

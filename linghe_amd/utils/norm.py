@@ -145,10 +145,14 @@ def triton_rms_norm_and_block_quant_forward(
 
     if M > 0:
         with torch.cuda.device(device):
+            ws, ws_bytes = (None, 0)
+            if output_mode == 2:
+                ws, ws_bytes = _lib.norm_workspace(x, M, n)
             _lib.check(_lib.lib.fq_rmsnorm_quant_fwd(
                 _lib.ptr(x), _lib.ptr(weight),
                 _lib.ptr(out) if output_mode != 1 else None,
                 _lib.ptr(scale) if output_mode != 1 else None,
                 _lib.ptr(rms), _lib.ptr(transpose_output), _lib.ptr(transpose_scale),
-                M, n, float(eps), int(bool(round_scale)), output_mode, kind, _lib.stream_of(x)))
+                M, n, float(eps), int(bool(round_scale)), output_mode, kind,
+                _lib.ptr(ws), ws_bytes, _lib.stream_of(x)))
     return out, scale, rms, transpose_output, transpose_scale
