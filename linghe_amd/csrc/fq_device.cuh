@@ -174,26 +174,20 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// sigmoid(x) = 1 / (1 + exp(-x)), each step good to ~1 ulp so that the result
-// agrees with a correctly rounded evaluation in ~95 % of the inputs:
-//   exp(-x) = exp2(t) * (1 + ln2 * lo),  t + lo = -x*log2(e) held as a
-//   double-float product (fp32 log2(e) alone is 1.3e-8 off), v_exp_f32 for exp2;
-//   the reciprocal is v_rcp_f32 plus one Newton step.
-// No range checks are needed: exp2 saturates to 0 / inf and 1/(1+inf) = 0.
+// sigmoid(x) = 1 / (1 + exp(-x)):
+//   exp(-x) = exp2(x * -log2(e)) with v_exp_f32 (1 ulp); the fp32 product costs up
+//   to |x|*4e-8 of relative error in exp(-x), which only matters where exp(-x) is
+//   large, i.e. where sigmoid (and silu) is small;
+//   the reciprocal is v_rcp_f32 plus one Newton step (correctly rounded but for
+//   ~1e-6 of the inputs).
+// The exponent is clamped so that 1 + exp(-x) stays finite: for x < -87 the result
+// is 2^-126 instead of 0, far below anything a code or a scale can see.
 __device__ __forceinline__ float sigmoid_f32(float x) {
-  const float c_hi = -1.4426950408889634f;     // -fp32(log2 e)
-  const float c_lo = -1.9259629911266175e-8f;   // -(log2 e - fp32(log2 e))
-  const float t = x * c_hi;
-  float lo = __builtin_fmaf(x, c_hi, -t);
-  lo = __builtin_fmaf(x, c_lo, lo);
-  const float e0 = __builtin_amdgcn_exp2f(t);
-  const float e = __builtin_fmaf(e0, lo * 0.6931471805599453f, e0);
-  const float d = 1.0f + e;
+  const float t = fminf(x * -1.4426950408889634f, 126.0f);
+  const float d = 1.0f + __builtin_amdgcn_exp2f(t);
   const float r0 = __builtin_amdgcn_rcpf(d);
   const float err = __builtin_fmaf(-d, r0, 1.0f);
-  const float r = __builtin_fmaf(err, r0, r0);
-  // exp overflow (x < -88.7): inf*lo and the Newton step make NaNs; the value is 1/(1+inf) = 0
-  return (e0 < 3.0e38f) ? r : 0.0f;
+  return __builtin_fmaf(err, r0, r0);
 }
 
 }  // namespace fq

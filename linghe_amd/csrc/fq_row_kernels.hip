@@ -53,6 +53,16 @@ __device__ __forceinline__ void load_row(const uint16_t* row, int n, uint4 (&raw
   }
 }
 
+// make the compiler forget what it knows about a packed row, so that the fp32
+// copies made before a reduction are not kept alive across it (they are cheap to
+// remake and cost four times the registers)
+template <int NCHUNK>
+__device__ __forceinline__ void forget(uint4 (&raw)[NCHUNK]) {
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k)
+    asm volatile("" : "+v"(raw[k].x), "+v"(raw[k].y), "+v"(raw[k].z), "+v"(raw[k].w));
+}
+
 __device__ __forceinline__ float rstd_from_sumsq(float ss, int n, float eps) {
   // rsqrt(sum/n + eps) as the fp32 CPU oracle evaluates it: true division,
   // correctly rounded sqrt, true reciprocal
@@ -162,7 +172,7 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
   int64_t r1 = r0 + rows_per_wg;
   if (r1 > M) r1 = M;
 
-  auto process = [&](const uint4 (&rx)[NCHUNK], const uint4 (&rg)[NCHUNK], int64_t row, int parity) {
+  auto process = [&](uint4 (&rx)[NCHUNK], uint4 (&rg)[NCHUNK], int64_t row, int parity) {
     // the sum of squares is taken exactly as the forward kernels take it, so that a
     // recomputed statistic equals a saved one bit for bit
     float ss = REUSE ? 0.f : sumsq<NCHUNK>(rx), dot = 0.f;
@@ -176,6 +186,8 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
       for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
     }
     block_sum2<T>(ss, dot, sh, parity);
+    forget<NCHUNK>(rx);
+    forget<NCHUNK>(rg);
     float r;
     if constexpr (REUSE) r = rstd_in[row];
     else r = rstd_from_sumsq(ss, n, eps);
@@ -227,20 +239,37 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
   }
 }
 
-// dgamma[c] = sum_p part[p, c], fixed order: 4 strided slices of p summed
-// sequentially, then combined 0..3.  64 columns per workgroup.
-__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ part, float* __restrict__ out,
-                                                     int P, int n) {
-  __shared__ float red[4][64];
-  const int col = blockIdx.x * 64 + (threadIdx.x & 63);
+// dgamma[c] = sum_p part[p, c] in a fixed order: 16 strided slices of p, each
+// summed sequentially (loads issued eight ahead), then combined 0..15.
+// 64 columns per workgroup of 1024 threads.
+constexpr int kColsumSlices = 16;
+__global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                      int P, int n) {
+  __shared__ float red[kColsumSlices][64];
+  const int lane = threadIdx.x & 63;
+  const int col = blockIdx.x * 64 + lane;
   const int slice = threadIdx.x >> 6;
   float acc = 0.f;
-  if (col < n)
-    for (int p = slice; p < P; p += 4) acc += part[(int64_t)p * n + col];
-  red[slice][threadIdx.x & 63] = acc;
+  if (col < n) {
+    const float* src = part + col;
+    int p = slice;
+    for (; p + 7 * kColsumSlices < P; p += 8 * kColsumSlices) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(p + u * kColsumSlices) * n];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; p < P; p += kColsumSlices) acc += src[(int64_t)p * n];
+  }
+  red[slice][lane] = acc;
   __syncthreads();
-  if (slice == 0 && col < n)
-    out[col] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+  if (slice == 0 && col < n) {
+    float tot = red[0][lane];
+#pragma unroll
+    for (int k = 1; k < kColsumSlices; ++k) tot += red[k][lane];
+    out[col] = tot;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -281,24 +310,21 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __rest
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
-// pick the workgroup width and chunks-per-thread for a row of n columns
+// Workgroup width and chunks-per-thread for a row of n columns.  Every kernel that
+// produces or recomputes the row statistic uses this one choice, so that the
+// statistic has the same bits wherever it is computed.
 static void pick_row_shape(int n, int& T, int& nchunk) {
   const int chunks = (n + 7) / 8;
-  T = 256;
-  if (chunks <= 64) T = 64;
-  else if (chunks <= 128) T = 128;
-  else if (chunks % 256 != 0 && chunks % 128 == 0 && chunks / 128 <= 8) T = 128;
+  T = chunks <= 64 ? 64 : (chunks <= 128 ? 128 : 256);
   nchunk = (chunks + T - 1) / T;
 }
 
 #define FQ_ROW_CASE(TT, NC, ...) \
   if (T == TT && nchunk == NC) { constexpr int kT = TT; constexpr int kNC = NC; __VA_ARGS__ } else
-#define FQ_ROW_SHAPES(...)                                                                               \
-  FQ_ROW_CASE(64, 1, __VA_ARGS__) FQ_ROW_CASE(128, 1, __VA_ARGS__) FQ_ROW_CASE(128, 2, __VA_ARGS__)      \
-  FQ_ROW_CASE(128, 3, __VA_ARGS__) FQ_ROW_CASE(128, 4, __VA_ARGS__) FQ_ROW_CASE(128, 5, __VA_ARGS__)     \
-  FQ_ROW_CASE(128, 6, __VA_ARGS__) FQ_ROW_CASE(128, 7, __VA_ARGS__) FQ_ROW_CASE(128, 8, __VA_ARGS__)     \
-  FQ_ROW_CASE(256, 1, __VA_ARGS__) FQ_ROW_CASE(256, 2, __VA_ARGS__) FQ_ROW_CASE(256, 3, __VA_ARGS__)     \
-  FQ_ROW_CASE(256, 4, __VA_ARGS__) { return hipErrorInvalidValue; }
+#define FQ_ROW_SHAPES(...)                                                                           \
+  FQ_ROW_CASE(64, 1, __VA_ARGS__) FQ_ROW_CASE(128, 1, __VA_ARGS__) FQ_ROW_CASE(256, 1, __VA_ARGS__)  \
+  FQ_ROW_CASE(256, 2, __VA_ARGS__) FQ_ROW_CASE(256, 3, __VA_ARGS__) FQ_ROW_CASE(256, 4, __VA_ARGS__) \
+  { return hipErrorInvalidValue; }
 
 hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* scale, float* rstd, int64_t M,
                               int n, float eps, int reuse_rstd, int quant, int round_scale, int kind,
@@ -351,7 +377,7 @@ hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, 
 #undef FQ_LAUNCH_BWD
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, stream, dg_part, dgamma, (int)P,
+  hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((n + 63) / 64)), dim3(1024), 0, stream, dg_part, dgamma, (int)P,
                      n);
   return hipGetLastError();
 }

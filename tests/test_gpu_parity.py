@@ -11,7 +11,7 @@ Acceptance (stricter than the reference's output_check):
     of sum(x^2) (RMSNorm) or on the exp implementation (SwiGLU), and dividing by
     448 can turn a 1-ulp difference of amax into 2 ulps of scale (the quotient's
     mantissa is 8/7 of the dividend's).
-      - SwiGLU family: >= 97 % within 1 ulp (96 % in the backward), none beyond
+      - SwiGLU family: >= 95 % within 1 ulp (94 % in the backward), none beyond
         8 ulp (a chain of six roundings after an exp that is itself good to
         1-2 ulp on either side), except that in the backward at most 0.5 % of
         the scales may differ by up to 1e-4 relative: dx1 = h*s + h*x1*(1-s)*s
@@ -34,8 +34,8 @@ from tests.helpers import (E4M3, E5M2, announce, check_quant_pair, gamma_bf16, g
 
 pytestmark = pytest.mark.gpu
 
-FUSED = dict(scale_max_ulp=8, scale_min_within1=0.97)                      # SwiGLU forward
-FUSED_BWD = dict(scale_max_ulp=8, scale_min_within1=0.96, outlier_rel=1e-4, outlier_frac=0.005)
+FUSED = dict(scale_max_ulp=8, scale_min_within1=0.95)                      # SwiGLU forward
+FUSED_BWD = dict(scale_max_ulp=8, scale_min_within1=0.94, outlier_rel=1e-4, outlier_frac=0.005)
 FUSED_NORM = dict(scale_max_ulp=8, scale_min_within1=0.9)                   # RMSNorm vs pure oracle
 EXACT = dict(scale_max_ulp=0, scale_min_within1=1.0, min_identical=1.0)
 
