@@ -89,9 +89,10 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
   const int tid = threadIdx.x;
   uint4 gm[NCHUNK];
   if constexpr (OUT != 2) load_row<T, NCHUNK>(gamma, n, gm);
-  const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
-  int64_t r1 = r0 + rows_per_wg;
-  if (r1 > M) r1 = M;
+  const int64_t G = gridDim.x;  // rows blockIdx.x, +G, +2G, ...
+  const int64_t r0 = blockIdx.x;
+  const int64_t r1 = M;
+  (void)rows_per_wg;
   if (r0 >= r1) return;
 
   auto process = [&](const uint4 (&raw)[NCHUNK], int64_t row, int parity) {
@@ -138,12 +139,12 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
 
   uint4 bufA[NCHUNK], bufB[NCHUNK];
   load_row<T, NCHUNK>(x + r0 * n, n, bufA);
-  for (int64_t row = r0; row < r1; row += 2) {
-    if (row + 1 < r1) load_row<T, NCHUNK>(x + (row + 1) * n, n, bufB);
+  for (int64_t row = r0; row < r1; row += 2 * G) {
+    if (row + G < r1) load_row<T, NCHUNK>(x + (row + G) * n, n, bufB);
     process(bufA, row, 0);
-    if (row + 1 < r1) {
-      if (row + 2 < r1) load_row<T, NCHUNK>(x + (row + 2) * n, n, bufA);
-      process(bufB, row + 1, 1);
+    if (row + G < r1) {
+      if (row + 2 * G < r1) load_row<T, NCHUNK>(x + (row + 2 * G) * n, n, bufA);
+      process(bufB, row + G, 1);
     }
   }
 }
@@ -168,9 +169,12 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[k][j] = 0.f;
 
-  const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
-  int64_t r1 = r0 + rows_per_wg;
-  if (r1 > M) r1 = M;
+  // rows blockIdx.x, blockIdx.x + G, blockIdx.x + 2G, ...: at any moment the
+  // workgroups of the grid work on neighbouring rows (one moving front in memory)
+  const int64_t G = gridDim.x;
+  const int64_t r0 = blockIdx.x;
+  const int64_t r1 = M;
+  (void)rows_per_wg;
 
   auto process = [&](uint4 (&rx)[NCHUNK], uint4 (&rg)[NCHUNK], int64_t row, int parity) {
     // the sum of squares is taken exactly as the forward kernels take it, so that a
@@ -208,22 +212,22 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
     }
   };
 
-  if (r0 < r1) {
+  if (r0 < r1) {  // the next row is prefetched into a second register set
     uint4 xa[NCHUNK], ga[NCHUNK], xb[NCHUNK], gb[NCHUNK];
     load_row<T, NCHUNK>(x + r0 * n, n, xa);
     load_row<T, NCHUNK>(dy + r0 * n, n, ga);
-    for (int64_t row = r0; row < r1; row += 2) {
-      if (row + 1 < r1) {
-        load_row<T, NCHUNK>(x + (row + 1) * n, n, xb);
-        load_row<T, NCHUNK>(dy + (row + 1) * n, n, gb);
+    for (int64_t row = r0; row < r1; row += 2 * G) {
+      if (row + G < r1) {
+        load_row<T, NCHUNK>(x + (row + G) * n, n, xb);
+        load_row<T, NCHUNK>(dy + (row + G) * n, n, gb);
       }
       process(xa, ga, row, 0);
-      if (row + 1 < r1) {
-        if (row + 2 < r1) {
-          load_row<T, NCHUNK>(x + (row + 2) * n, n, xa);
-          load_row<T, NCHUNK>(dy + (row + 2) * n, n, ga);
+      if (row + G < r1) {
+        if (row + 2 * G < r1) {
+          load_row<T, NCHUNK>(x + (row + 2 * G) * n, n, xa);
+          load_row<T, NCHUNK>(dy + (row + 2 * G) * n, n, ga);
         }
-        process(xb, gb, row + 1, 1);
+        process(xb, gb, row + G, 1);
       }
     }
   }
