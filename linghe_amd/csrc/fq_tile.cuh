@@ -58,33 +58,62 @@ __device__ __forceinline__ float max_across_rows(float v) {
   return fmaxf(as_f32(b[0]), as_f32(b[1]));
 }
 
-// store up to 16 transposed code bytes; `n` of them are valid rows
-__device__ __forceinline__ void store_t_chunk(uint8_t* dst, const uint4& v, int n) {
-  if (n <= 0) return;
-  uintptr_t a = (uintptr_t)dst;
-  if (n >= 16 && (a & 15) == 0) {
-    *(uint4*)dst = v;
-    return;
-  }
-  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-  if ((a & 3) == 0) {
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      if (4 * d + 4 <= n) {
-        ((uint32_t*)dst)[d] = w[d];
-      } else {
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          if (4 * d + b < n) dst[4 * d + b] = (uint8_t)(w[d] >> (8 * b));
-      }
-    }
+// Write the first `len` bytes of one transposed row from LDS (`lds_row`: 128 bytes
+// as eight 16-byte chunks, chunk k stored at position k ^ swz) to the byte address
+// `dst_row`, which may have ANY alignment (per-expert transposed rows are packed
+// back to back with a stride of count_e bytes).  Called by the 8 threads
+// ch = 0..7 that share the row.  The row is cut at the 16-byte boundaries of the
+// DESTINATION: destination chunk m holds source bytes [16m - a, 16m - a + 16),
+// a = dst_row & 15, assembled from the two source chunks around it with dword
+// selects and v_alignbyte; whole chunks leave as one 16-byte store, the (at most
+// two) ragged ends as dword / byte stores of exactly the bytes of this row.
+__device__ __forceinline__ void store_t_dword(uint8_t* dst, int d, uint32_t val, int j0, int j1) {
+  if (4 * d >= j0 && 4 * d + 4 <= j1) {
+    ((uint32_t*)dst)[d] = val;
   } else {
 #pragma unroll
-    for (int d = 0; d < 4; ++d)
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-        if (4 * d + b < n) dst[4 * d + b] = (uint8_t)(w[d] >> (8 * b));
+    for (int b = 0; b < 4; ++b)
+      if (4 * d + b >= j0 && 4 * d + b < j1) dst[4 * d + b] = (uint8_t)(val >> (8 * b));
   }
+}
+
+__device__ __forceinline__ void store_t_chunk(const uint8_t* lds_row, int swz, uint8_t* dst0, int a, int len, int m) {
+  const int s0 = 16 * m - a;  // source index of destination byte 0 of this chunk
+  if (s0 >= len) return;
+  uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
+  if (m >= 1) lo = *(const uint4*)(lds_row + (((m - 1) ^ swz) * 16));
+  if (m <= 7) hi = *(const uint4*)(lds_row + ((m ^ swz) * 16));
+  // window bytes 0..31 = source bytes 16(m-1) .. 16(m+1); destination byte j = window byte 16 - a + j
+  const int sb = 16 - a;  // 1..16
+  const bool b0 = (sb >> 2) & 1, b1 = (sb >> 3) & 1;
+  const uint32_t u0 = b0 ? lo.y : lo.x, u1 = b0 ? lo.z : lo.y, u2 = b0 ? lo.w : lo.z, u3 = b0 ? hi.x : lo.w;
+  const uint32_t u4 = b0 ? hi.y : hi.x, u5 = b0 ? hi.z : hi.y, u6 = b0 ? hi.w : hi.z;
+  const uint32_t t0 = b1 ? u2 : u0, t1 = b1 ? u3 : u1, t2 = b1 ? u4 : u2, t3 = b1 ? u5 : u3, t4 = b1 ? u6 : u4;
+  const uint32_t rs = (uint32_t)(sb & 3);
+  const bool al = a == 0;
+  const uint32_t o0 = al ? hi.x : __builtin_amdgcn_alignbyte(t1, t0, rs);
+  const uint32_t o1 = al ? hi.y : __builtin_amdgcn_alignbyte(t2, t1, rs);
+  const uint32_t o2 = al ? hi.z : __builtin_amdgcn_alignbyte(t3, t2, rs);
+  const uint32_t o3 = al ? hi.w : __builtin_amdgcn_alignbyte(t4, t3, rs);
+  const int j0 = s0 < 0 ? -s0 : 0;                   // first valid destination byte
+  const int j1 = (len - s0) < 16 ? (len - s0) : 16;  // one past the last valid one
+  uint8_t* dst = dst0 + 16 * m;
+  if (j0 == 0 && j1 == 16) {
+    *(uint4*)dst = make_uint4(o0, o1, o2, o3);
+  } else {
+    store_t_dword(dst, 0, o0, j0, j1);
+    store_t_dword(dst, 1, o1, j0, j1);
+    store_t_dword(dst, 2, o2, j0, j1);
+    store_t_dword(dst, 3, o3, j0, j1);
+  }
+}
+
+__device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uint8_t* dst_row, int len, int ch) {
+  const int a = (int)((uintptr_t)dst_row & 15u);
+  uint8_t* dst0 = dst_row - a;
+  store_t_chunk(lds_row, swz, dst0, a, len, ch);
+  // a ninth destination chunk exists when a misaligned row runs past 8 * 16 bytes
+  if (ch == 0 && a + len > 128) store_t_chunk(lds_row, swz, dst0, a, len, 8);
 }
 
 // Quantise the tile held in registers (v[s][j] = element (rg*RPT+s, cg*8+j);
@@ -206,10 +235,12 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
 #pragma unroll
     for (int k = 0; k < kGroup / kRowsPerPass; ++k) {
       const int c = (tid >> 3) + k * kRowsPerPass;
-      const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
-      uint8_t* dst = o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16;
-      if constexpr (FULL) *(uint4*)dst = val;
-      else store_t_chunk(dst, val, o.rows_valid - ch * 16);
+      if constexpr (FULL) {
+        const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
+        *(uint4*)(o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16) = val;
+      } else {
+        store_t_row(sh.t + c * kGroup, (c >> 3) & 7, o.qt + o.t_off + (int64_t)c * o.t_ld, o.rows_valid, ch);
+      }
     }
     __syncthreads();  // LDS is reused by a following call
   }
@@ -237,7 +268,7 @@ struct ExpertTile {
 };
 
 struct ExpertScanShared {
-  long long wave_rows[16];
+  int wave_rows[16];
   int wave_blocks[16];
   ExpertTile found;
 };
@@ -246,10 +277,23 @@ __device__ __forceinline__ int load_count(const void* counts, int is_i64, int e)
   return is_i64 ? (int)((const long long*)counts)[e] : ((const int*)counts)[e];
 }
 
+// inclusive prefix sum over the 64 lanes of a wave with DPP row shifts and the two
+// row broadcasts (no LDS traffic, ~6 dependent VALU steps)
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
+  return v;
+}
+
 // Which expert owns the global 128-row block `blk` (blocks are numbered expert
 // after expert, ceil(count/128) per expert)?  Computed from the device-side
-// counts by a block-wide prefix scan; every thread returns the same answer.
-// An out-of-range blk (host/device counts disagree) yields expert = -1.
+// counts by a workgroup-wide prefix scan, THREADS experts per step; every thread
+// returns the same answer.  An out-of-range blk (host and device counts
+// disagree) yields expert = -1.
 template <int THREADS>
 __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int is_i64, int n_experts,
                                                        int blk, ExpertScanShared& sh) {
@@ -258,31 +302,20 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
   const int wave = tid >> 6;
   constexpr int kWaves = THREADS / 64;
   if (tid == 0) sh.found.expert = -1;
-  long long run_rows = 0;
-  int run_blocks = 0;
+  int run_rows = 0, run_blocks = 0;
   for (int base = 0; base < n_experts; base += THREADS) {
     const int e = base + tid;
     const int c = (e < n_experts) ? load_count(counts, is_i64, e) : 0;
     const int nb = (c + kGroup - 1) / kGroup;
-    long long rows = c;
-    int blocks = nb;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const long long r2 = __shfl_up(rows, d, 64);
-      const int b2 = __shfl_up(blocks, d, 64);
-      if (lane >= d) { rows += r2; blocks += b2; }
-    }
-    __syncthreads();  // previous iteration's readers are done
+    const int rows = wave_inclusive_scan(c);
+    const int blocks = wave_inclusive_scan(nb);
+    if (base != 0) __syncthreads();  // readers of the previous step are done
     if (lane == 63) { sh.wave_rows[wave] = rows; sh.wave_blocks[wave] = blocks; }
     __syncthreads();
-    long long rows_before = run_rows;
-    int blocks_before = run_blocks;
-    long long tot_rows = 0;
-    int tot_blocks = 0;
+    int rows_before = run_rows, blocks_before = run_blocks, tot_rows = 0, tot_blocks = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-      const long long wr = sh.wave_rows[w];
-      const int wb = sh.wave_blocks[w];
+      const int wr = sh.wave_rows[w], wb = sh.wave_blocks[w];
       if (w < wave) { rows_before += wr; blocks_before += wb; }
       tot_rows += wr;
       tot_blocks += wb;
@@ -293,16 +326,16 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
       t.expert = e;
       t.count = c;
       t.rb = blk - excl_blocks;
-      t.row_start = rows_before + rows - c;
+      t.row_start = (int64_t)(rows_before + rows - c);
       t.tblock_start = excl_blocks;
       sh.found = t;
     }
     run_rows += tot_rows;
     run_blocks += tot_blocks;
-    if (blk < run_blocks) break;  // uniform: found in this chunk
+    if (blk < run_blocks) break;  // uniform: found in this step
   }
   __syncthreads();
-  ExpertTile out = sh.found;
+  const ExpertTile out = sh.found;
   __syncthreads();
   return out;
 }
