@@ -29,7 +29,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-TWO_PASS = False  # --two-pass: RMSNorm+quant mode 2 without the workspace (statistic kernel + tile kernel)
+SINGLE_PASS_CASES = {"cfg1_single"}  # RMSNorm+quant mode 2 with the workspace (one pass over x)
 INFINITY_CACHE_BYTES = 256 << 20
 FP8 = torch.float8_e4m3fn
 
@@ -85,7 +85,7 @@ def build_cases(names, dev):
                 s["st"] = torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32)
             else:
                 s["qt"], s["st"] = None, None
-            ws, ws_bytes = _lib.norm_workspace(s["x"], M, n) if (mode == 2 and not TWO_PASS) else (None, 0)
+            ws, ws_bytes = _lib.norm_workspace(s["x"], M, n) if name in SINGLE_PASS_CASES else (None, 0)
             s["args"] = (_p(s["x"]), _p(gd), _p(s["q"]), _p(s["s"]), _p(s["rstd"]), _p(s["qt"]), _p(s["st"]),
                          M, n, float(eps), 0, mode, _lib.FQ_E4M3, _p(ws), ws_bytes, stream)
             return s
@@ -97,7 +97,10 @@ def build_cases(names, dev):
             from oracle import fq_oracle as O
             return O.rms_norm_and_block_quant_forward(x_cpu, g_cpu, eps, False)
 
-        return Case(name, "triton_rms_norm_and_block_quant_forward(output_mode=%d)" % mode, [M, n],
+        label = "triton_rms_norm_and_block_quant_forward(output_mode=%d)" % mode
+        if mode == 2:
+            label += " single pass" if name in SINGLE_PASS_CASES else " two passes"
+        return Case(name, label, [M, n],
                     configs.bytes_rmsnorm_quant(M, n, mode), make_set, launch, cpu_fn)
 
     lazy = {}
@@ -108,6 +111,7 @@ def build_cases(names, dev):
         return lazy["cfg5"]
 
     add("cfg1", build=lambda: rms_quant_case("cfg1", configs.cfg1_rmsnorm_quant(), 2))
+    add("cfg1_single", build=lambda: rms_quant_case("cfg1_single", configs.cfg1_rmsnorm_quant(), 2))
     add("cfg5b", build=lambda: rms_quant_case("cfg5b", cfg5(), 2))
     add("cfg5c", build=lambda: rms_quant_case("cfg5c", cfg5(), 1))
 
@@ -301,7 +305,7 @@ def time_cpu(case, budget_s):
     return best * 1e6, len(runs)
 
 
-ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c"]
+ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c"]
 
 
 def main():
@@ -315,8 +319,6 @@ def main():
     ap.add_argument("--no-headline", action="store_true",
                     help="profiling aid: run only the named configs and print their results without the headline line")
     ap.add_argument("--hot-only", action="store_true", help="profiling aid: one buffer set, no rotation")
-    ap.add_argument("--two-pass", action="store_true",
-                    help="run RMSNorm+quant mode 2 as statistic kernel + tile kernel (no workspace)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (every row block / expert is independent, "
@@ -325,8 +327,6 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
-    global TWO_PASS
-    TWO_PASS = args.two_pass
     names = ALL if args.configs == "all" else [c.strip() for c in args.configs.split(",")]
     if "cfg1" not in names and not args.no_headline:
         names = ["cfg1"] + names

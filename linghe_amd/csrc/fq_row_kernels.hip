@@ -177,8 +177,6 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
   (void)rows_per_wg;
 
   auto process = [&](uint4 (&rx)[NCHUNK], uint4 (&rg)[NCHUNK], int64_t row, int parity) {
-    // the sum of squares is taken exactly as the forward kernels take it, so that a
-    // recomputed statistic equals a saved one bit for bit
     float ss = REUSE ? 0.f : sumsq<NCHUNK>(rx), dot = 0.f;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
@@ -314,32 +312,40 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __rest
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
-// Workgroup width and chunks-per-thread for a row of n columns.  Every kernel that
-// produces or recomputes the row statistic uses this one choice, so that the
-// statistic has the same bits wherever it is computed.
-static void pick_row_shape(int n, int& T, int& nchunk) {
+// Forward kernels: one wave per row (64-thread workgroups, no barrier), every load
+// of a row in flight at once and the next row prefetched.
+// Backward kernel: 256 threads per row (it also carries the dgamma accumulators).
+static void pick_row_shape(int n, int T, int& nchunk) {
   const int chunks = (n + 7) / 8;
-  T = chunks <= 64 ? 64 : (chunks <= 128 ? 128 : 256);
   nchunk = (chunks + T - 1) / T;
 }
 
 #define FQ_ROW_CASE(TT, NC, ...) \
-  if (T == TT && nchunk == NC) { constexpr int kT = TT; constexpr int kNC = NC; __VA_ARGS__ } else
-#define FQ_ROW_SHAPES(...)                                                                           \
-  FQ_ROW_CASE(64, 1, __VA_ARGS__) FQ_ROW_CASE(128, 1, __VA_ARGS__) FQ_ROW_CASE(256, 1, __VA_ARGS__)  \
-  FQ_ROW_CASE(256, 2, __VA_ARGS__) FQ_ROW_CASE(256, 3, __VA_ARGS__) FQ_ROW_CASE(256, 4, __VA_ARGS__) \
-  { return hipErrorInvalidValue; }
+  if (nchunk == NC) { constexpr int kT = TT; constexpr int kNC = NC; __VA_ARGS__ } else
+#define FQ_FWD_SHAPES(...)                                                                         \
+  FQ_ROW_CASE(64, 1, __VA_ARGS__) FQ_ROW_CASE(64, 2, __VA_ARGS__) FQ_ROW_CASE(64, 3, __VA_ARGS__)  \
+  FQ_ROW_CASE(64, 4, __VA_ARGS__) FQ_ROW_CASE(64, 5, __VA_ARGS__) FQ_ROW_CASE(64, 6, __VA_ARGS__)  \
+  FQ_ROW_CASE(64, 7, __VA_ARGS__) FQ_ROW_CASE(64, 8, __VA_ARGS__) FQ_ROW_CASE(64, 9, __VA_ARGS__)  \
+  FQ_ROW_CASE(64, 10, __VA_ARGS__) FQ_ROW_CASE(64, 11, __VA_ARGS__) FQ_ROW_CASE(64, 12, __VA_ARGS__) \
+  FQ_ROW_CASE(64, 13, __VA_ARGS__) FQ_ROW_CASE(64, 14, __VA_ARGS__) FQ_ROW_CASE(64, 15, __VA_ARGS__) \
+  FQ_ROW_CASE(64, 16, __VA_ARGS__) { return hipErrorInvalidValue; }
+#define FQ_BWD_SHAPES(...)                                                                           \
+  FQ_ROW_CASE(256, 1, __VA_ARGS__) FQ_ROW_CASE(256, 2, __VA_ARGS__) FQ_ROW_CASE(256, 3, __VA_ARGS__) \
+  FQ_ROW_CASE(256, 4, __VA_ARGS__) { return hipErrorInvalidValue; }
 
 hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* scale, float* rstd, int64_t M,
                               int n, float eps, int reuse_rstd, int quant, int round_scale, int kind,
                               hipStream_t stream) {
   if (M == 0) return hipSuccess;
-  int T, nchunk;
-  pick_row_shape(n, T, nchunk);
-  const int rows_per_wg = 16;
-  const dim3 grid((unsigned)((M + rows_per_wg - 1) / rows_per_wg));
+  int nchunk;
+  pick_row_shape(n, 64, nchunk);
+  const int rows_per_wg = 1;
+  // one wave per workgroup; at most 32 of them per CU, rows beyond that by striding
+  int64_t wgs = M;
+  if (wgs > 256 * 32) wgs = 256 * 32;
+  const dim3 grid((unsigned)wgs);
 #define FQ_LAUNCH_FWD(REUSE, QUANT, KINDV, ROUNDV)                                                          \
-  FQ_ROW_SHAPES(hipLaunchKernelGGL((rmsnorm_fwd_kernel<kT, kNC, REUSE, QUANT, KINDV, ROUNDV>), grid,       \
+  FQ_FWD_SHAPES(hipLaunchKernelGGL((rmsnorm_fwd_kernel<kT, kNC, REUSE, QUANT, KINDV, ROUNDV>), grid,       \
                                    dim3(kT), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, out,   \
                                    scale, rstd, M, n, eps, rows_per_wg);)
   // quant: 0 = bf16 output, 1 = fp8 codes + scales, 2 = statistic only
@@ -368,13 +374,13 @@ int64_t rmsnorm_bwd_partials(int64_t M) {
 hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
                               float* dgamma, float* dg_part, int64_t n_partials, int64_t M, int n, float eps,
                               hipStream_t stream) {
-  int T, nchunk;
-  pick_row_shape(n, T, nchunk);
+  int nchunk;
+  pick_row_shape(n, 256, nchunk);
   const int64_t P = n_partials;
   const int rows_per_wg = (int)((M + P - 1) / P);
   const dim3 grid((unsigned)P);
 #define FQ_LAUNCH_BWD(REUSE)                                                                               \
-  FQ_ROW_SHAPES(hipLaunchKernelGGL((rmsnorm_bwd_kernel<kT, kNC, REUSE>), grid, dim3(kT), 0, stream,        \
+  FQ_BWD_SHAPES(hipLaunchKernelGGL((rmsnorm_bwd_kernel<kT, kNC, REUSE>), grid, dim3(kT), 0, stream,        \
                                    (const uint16_t*)dy, (const uint16_t*)x, (const uint16_t*)gamma, rstd,  \
                                    (uint16_t*)dx, dg_part, M, n, eps, rows_per_wg);)
   if (rstd) { FQ_LAUNCH_BWD(true) } else { FQ_LAUNCH_BWD(false) }

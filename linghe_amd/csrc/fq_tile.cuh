@@ -67,13 +67,33 @@ __device__ __forceinline__ float max_across_rows(float v) {
 // a = dst_row & 15, assembled from the two source chunks around it with dword
 // selects and v_alignbyte; whole chunks leave as one 16-byte store, the (at most
 // two) ragged ends as dword / byte stores of exactly the bytes of this row.
-__device__ __forceinline__ void store_t_dword(uint8_t* dst, int d, uint32_t val, int j0, int j1) {
-  if (4 * d >= j0 && 4 * d + 4 <= j1) {
-    ((uint32_t*)dst)[d] = val;
+// dword k (k = 0..3, lane-variable) of a 16-byte chunk held in four registers
+__device__ __forceinline__ uint32_t pick_dword(uint32_t o0, uint32_t o1, uint32_t o2, uint32_t o3, int k) {
+  const uint32_t lo = (k & 1) ? o1 : o0;
+  const uint32_t hi = (k & 1) ? o3 : o2;
+  return (k & 2) ? hi : lo;
+}
+
+// Store destination bytes [j0, j1) of the 16-byte aligned chunk at dst.
+// A ragged head (j1 == 16) or tail (j0 == 0) leaves as at most one byte, one
+// short, one dword and one qword store, each naturally aligned; a chunk ragged at
+// both ends (a row shorter than 16 bytes) goes byte by byte.
+__device__ __forceinline__ void store_t_partial(uint8_t* dst, uint32_t o0, uint32_t o1, uint32_t o2, uint32_t o3,
+                                                int j0, int j1) {
+  if (j1 == 16) {  // head: valid bytes j0..15
+    int p = j0;
+    if (p & 1) { dst[p] = (uint8_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); p += 1; }
+    if (p & 2) { *(uint16_t*)(dst + p) = (uint16_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); p += 2; }
+    if (p & 4) { *(uint32_t*)(dst + p) = pick_dword(o0, o1, o2, o3, p >> 2); p += 4; }
+    if (p & 8) { *(uint2*)(dst + 8) = make_uint2(o2, o3); }
+  } else if (j0 == 0) {  // tail: valid bytes 0..j1-1
+    int p = 0;
+    if (j1 & 8) { *(uint2*)dst = make_uint2(o0, o1); p = 8; }
+    if (j1 & 4) { *(uint32_t*)(dst + p) = pick_dword(o0, o1, o2, o3, p >> 2); p += 4; }
+    if (j1 & 2) { *(uint16_t*)(dst + p) = (uint16_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); p += 2; }
+    if (j1 & 1) { dst[p] = (uint8_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); }
   } else {
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-      if (4 * d + b >= j0 && 4 * d + b < j1) dst[4 * d + b] = (uint8_t)(val >> (8 * b));
+    for (int j = j0; j < j1; ++j) dst[j] = (uint8_t)(pick_dword(o0, o1, o2, o3, j >> 2) >> (8 * (j & 3)));
   }
 }
 
@@ -101,10 +121,7 @@ __device__ __forceinline__ void store_t_chunk(const uint8_t* lds_row, int swz, u
   if (j0 == 0 && j1 == 16) {
     *(uint4*)dst = make_uint4(o0, o1, o2, o3);
   } else {
-    store_t_dword(dst, 0, o0, j0, j1);
-    store_t_dword(dst, 1, o1, j0, j1);
-    store_t_dword(dst, 2, o2, j0, j1);
-    store_t_dword(dst, 3, o3, j0, j1);
+    store_t_partial(dst, o0, o1, o2, o3, j0, j1);
   }
 }
 

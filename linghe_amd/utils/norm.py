@@ -13,6 +13,14 @@ from .. import _lib
 
 _MAX_HIDDEN = 8192  # the reference asserts next_power_of_2(n) <= 8192
 
+# output_mode 2 of triton_rms_norm_and_block_quant_forward:
+#   False  two passes (row statistic, then the tile kernel): the fastest measured
+#          variant on MI355X at every size tried;
+#   True   hand the library its workspace, so that problems of at most 1024 tiles
+#          run as ONE pass over x (the statistic is exchanged between workgroups
+#          inside the kernel): algorithmic HBM traffic, ~8 % slower at 8192x2048.
+SINGLE_PASS = False
+
 
 def _rows_cols(x):
     shape = x.shape
@@ -146,7 +154,7 @@ def triton_rms_norm_and_block_quant_forward(
     if M > 0:
         with torch.cuda.device(device):
             ws, ws_bytes = (None, 0)
-            if output_mode == 2:
+            if output_mode == 2 and SINGLE_PASS:
                 ws, ws_bytes = _lib.norm_workspace(x, M, n)
             _lib.check(_lib.lib.fq_rmsnorm_quant_fwd(
                 _lib.ptr(x), _lib.ptr(weight),

@@ -171,9 +171,12 @@ def test_rmsnorm_fwd_bwd(gpu, M, N):
     assert dw.dtype == torch.float32 and dw.shape == (N,)
     check_bf16("rmsnorm.dx", dx_ref, dx)
     torch.testing.assert_close(dw.cpu(), dw_ref, rtol=2e-4, atol=2e-4 * float(dw_ref.abs().max()))
+    # with a saved statistic (its last bit may differ from the one the backward
+    # recomputes: the forward adds the squares in another order)
     dx2, dw2 = triton_rms_norm_backward(dyd, xd, wd, rms=rms)
     torch.cuda.synchronize()
-    assert torch.equal(dx2.cpu(), dx.cpu()) and torch.equal(dw2.cpu(), dw.cpu())
+    check_bf16("rmsnorm.dx(rms given)", dx_ref, dx2)
+    torch.testing.assert_close(dw2.cpu(), dw_ref, rtol=2e-4, atol=2e-4 * float(dw_ref.abs().max()))
     # 3-D input
     if M % 4 == 0:
         y3, _ = triton_rms_norm_forward(xd.view(4, M // 4, N), wd)
@@ -210,7 +213,7 @@ def test_rmsnorm_and_block_quant(gpu, M, N, round_scale):
     check_quant_pair("rms.1.col", qt_ref, st_ref, qt, st, **kw)
     q2, s2, rms2, qt2, st2 = fwd(xd, wd, round_scale=round_scale, output_mode=2)
     torch.cuda.synchronize()
-    # mode 0 (row kernel) and mode 2 (single-pass tile kernel) add the squares in a different order
+    # mode 0 and mode 2 agree in the statistic (same statistic kernel arithmetic)
     C.assert_scales(rms.cpu(), rms2.cpu(), "rstd mode0 vs mode2", max_ulp=4, min_within_1ulp=0.9)
     C.assert_scales(r_ref, rms2.cpu(), "rstd2", max_ulp=4, min_within_1ulp=0.9)
     check_quant_pair("rms.2.row", q_ref, s_ref, q2, s2, **kw)
@@ -222,10 +225,21 @@ def test_rmsnorm_and_block_quant(gpu, M, N, round_scale):
     p_ref = O.rms_norm_and_block_quant_forward(x, w, round_scale=round_scale, rstd=rms2.cpu())
     check_quant_pair("rms.pinned.row", p_ref[0], p_ref[1], q2, s2, **EXACT)
     check_quant_pair("rms.pinned.col", p_ref[3], p_ref[4], qt2, st2, **EXACT)
-    # repeated calls reuse the workspace (entries are stamped per call, nothing is cleared)
-    q3, s3, rms3, qt3, st3 = fwd(xd, wd, round_scale=round_scale, output_mode=2)
-    torch.cuda.synchronize()
-    for a, b in ((q2, q3), (s2, s3), (rms2, rms3), (qt2, qt3), (st2, st3)):
+    # single-pass variant (opt-in): same rule; repeated calls reuse the workspace
+    # (entries are stamped per call, nothing is cleared)
+    import linghe_amd.utils.norm as norm_mod
+    norm_mod.SINGLE_PASS = True
+    try:
+        q3, s3, rms3, qt3, st3 = fwd(xd, wd, round_scale=round_scale, output_mode=2)
+        q4, s4, rms4, qt4, st4 = fwd(xd, wd, round_scale=round_scale, output_mode=2)
+        torch.cuda.synchronize()
+    finally:
+        norm_mod.SINGLE_PASS = False
+    C.assert_scales(r_ref, rms3.cpu(), "rstd (single pass)", max_ulp=4, min_within_1ulp=0.9)
+    p_ref = O.rms_norm_and_block_quant_forward(x, w, round_scale=round_scale, rstd=rms3.cpu())
+    check_quant_pair("rms.single.row", p_ref[0], p_ref[1], q3, s3, **EXACT)
+    check_quant_pair("rms.single.col", p_ref[3], p_ref[4], qt3, st3, **EXACT)
+    for a, b in ((q3, q4), (s3, s4), (rms3, rms4), (qt3, qt4), (st3, st4)):
         assert torch.equal(a.view(torch.uint8).cpu(), b.view(torch.uint8).cpu())
 
 
@@ -244,15 +258,21 @@ def test_rmsnorm_quant_single_pass_wait_bound(gpu):
     x = randn_bf16(g, M, N)
     w = gamma_bf16(g, N)
     xd, wd = _dev(x, gpu), _dev(w, gpu)
-    base = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
-    torch.cuda.synchronize()
+    import linghe_amd.utils.norm as norm_mod
+    norm_mod.SINGLE_PASS = True
     try:
-        _lib.lib.fq_set_wait_limit(1)
-        short = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
+        base = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
+        torch.cuda.synchronize()
+        try:
+            _lib.lib.fq_set_wait_limit(1)
+            short = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
+            torch.cuda.synchronize()
+        finally:
+            _lib.lib.fq_set_wait_limit(0)
+        again = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
         torch.cuda.synchronize()
     finally:
-        _lib.lib.fq_set_wait_limit(0)
-    again = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
+        norm_mod.SINGLE_PASS = False
     for a, b, c in zip(base, short, again):
         assert torch.equal(a, b) and torch.equal(a, c)
     # two-pass path through the C ABI (no workspace)
