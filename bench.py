@@ -305,6 +305,13 @@ def time_cpu(case, budget_s):
     return best * 1e6, len(runs)
 
 
+# HBM bytes per call of the headline entry point (statistic kernel + tile kernel),
+# from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
+# counters read for the 256 MiB `copy` case (x2.0 and x1.0):
+# fetched 33.63 + 33.99 MB, written 0.26 + 34.60 MB; algorithmic bytes are 68.19 MB,
+# the difference is the second read of x.
+CFG1_MEASURED_TRAFFIC_BYTES = 102.48e6
+
 ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c"]
 
 
@@ -383,7 +390,7 @@ def main():
                                "output_mode 2, round_scale False, buffers rotated beyond the Infinity Cache",
                    "entry": head["entry"]},
         "roofline": {"bound": "hbm", "achieved": head["gb_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["frac_of_hbm_peak"], "traffic": None},
+                     "frac": head["frac_of_hbm_peak"], "traffic": CFG1_MEASURED_TRAFFIC_BYTES},
         "configs": results,
     }
     if headline_cpu is not None:

@@ -174,6 +174,25 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// the same for a double (two dwords per DPP move): used where a sum has to come
+// out independent of the order of its terms
+template <int CTRL>
+__device__ __forceinline__ double dpp_mov_d(double v) {
+  const uint64_t u = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)u, CTRL, 0xf, 0xf, true);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)(u >> 32), CTRL, 0xf, 0xf, true);
+  return __builtin_bit_cast(double, (uint64_t)lo | ((uint64_t)hi << 32));
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+  v += dpp_mov_d<kDppQuadXor1>(v);
+  v += dpp_mov_d<kDppQuadXor2>(v);
+  v += dpp_mov_d<kDppRowHalfMirror>(v);
+  v += dpp_mov_d<kDppRowMirror>(v);
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
 // sigmoid(x) = 1 / (1 + exp(-x)):
 //   exp(-x) = exp2(x * -log2(e)) with v_exp_f32 (1 ulp); the fp32 product costs up
 //   to |x|*4e-8 of relative error in exp(-x), which only matters where exp(-x) is

@@ -19,6 +19,7 @@ namespace fq {
 template <int T>
 struct RowShared {
   float red[2][2][T / 64];  // [parity][value][wave]
+  double redd[2][T / 64];   // [parity][wave]
 };
 
 // sum of (a, b) over the workgroup, fixed order; one barrier per call
@@ -38,6 +39,28 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, RowShared<T>& sh,
 #pragma unroll
     for (int w = 1; w < T / 64; ++w) {
       a += sh.red[parity][0][w];
+      b += sh.red[parity][1][w];
+    }
+  }
+}
+
+// the same with the first value a double
+template <int T>
+__device__ __forceinline__ void block_sum2(double& a, float& b, RowShared<T>& sh, int parity) {
+  a = wave_sum_d(a);
+  b = wave_sum(b);
+  if constexpr (T > 64) {
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+      sh.redd[parity][wave] = a;
+      sh.red[parity][1][wave] = b;
+    }
+    __syncthreads();
+    a = sh.redd[parity][0];
+    b = sh.red[parity][1][0];
+#pragma unroll
+    for (int w = 1; w < T / 64; ++w) {
+      a += sh.redd[parity][w];
       b += sh.red[parity][1][w];
     }
   }
@@ -69,11 +92,17 @@ __device__ __forceinline__ float rstd_from_sumsq(float ss, int n, float eps) {
   return 1.0f / sqrtf(ss / (float)n + eps);
 }
 
+// the thread's share of a row's sum of squares: every aligned group of 8 elements
+// is summed in fp32 in a fixed order (exact products), the groups are added in
+// double.  The row total then does not depend on how the groups are split over
+// lanes and waves, so every kernel that computes the statistic (forward,
+// backward, any row shape) gets the same fp32 value: the exact sum of the group
+// sums, rounded once
 template <int NCHUNK>
-__device__ __forceinline__ float sumsq(const uint4 (&raw)[NCHUNK]) {
-  float ss = 0.f;
+__device__ __forceinline__ double sumsq(const uint4 (&raw)[NCHUNK]) {
+  double ss = 0.0;
 #pragma unroll
-  for (int k = 0; k < NCHUNK; ++k) ss += sumsq8(raw[k]);
+  for (int k = 0; k < NCHUNK; ++k) ss += (double)sumsq8(raw[k]);
   return ss;
 }
 
@@ -100,9 +129,10 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
     if constexpr (REUSE) {
       r = rstd[row];
     } else {
-      float ss = sumsq<NCHUNK>(raw), dummy = 0.f;
+      double ss = sumsq<NCHUNK>(raw);
+      float dummy = 0.f;
       block_sum2<T>(ss, dummy, sh, parity);
-      r = rstd_from_sumsq(ss, n, eps);
+      r = rstd_from_sumsq((float)ss, n, eps);
       if (tid == 0) rstd[row] = r;
     }
     if constexpr (OUT == 2) return;
@@ -177,7 +207,9 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
   (void)rows_per_wg;
 
   auto process = [&](uint4 (&rx)[NCHUNK], uint4 (&rg)[NCHUNK], int64_t row, int parity) {
-    float ss = REUSE ? 0.f : sumsq<NCHUNK>(rx), dot = 0.f;
+    double ss = 0.0;
+    if constexpr (!REUSE) ss = sumsq<NCHUNK>(rx);
+    float dot = 0.f;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
       float a[8], g[8], w[8];
@@ -187,12 +219,17 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
 #pragma unroll
       for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
     }
-    block_sum2<T>(ss, dot, sh, parity);
+    if constexpr (REUSE) {
+      float unused = 0.f;
+      block_sum2<T>(unused, dot, sh, parity);
+    } else {
+      block_sum2<T>(ss, dot, sh, parity);
+    }
     forget<NCHUNK>(rx);
     forget<NCHUNK>(rg);
     float r;
     if constexpr (REUSE) r = rstd_in[row];
-    else r = rstd_from_sumsq(ss, n, eps);
+    else r = rstd_from_sumsq((float)ss, n, eps);
     const float coef = ((r * r) * r) * dot / (float)n;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {

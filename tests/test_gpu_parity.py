@@ -171,12 +171,13 @@ def test_rmsnorm_fwd_bwd(gpu, M, N):
     assert dw.dtype == torch.float32 and dw.shape == (N,)
     check_bf16("rmsnorm.dx", dx_ref, dx)
     torch.testing.assert_close(dw.cpu(), dw_ref, rtol=2e-4, atol=2e-4 * float(dw_ref.abs().max()))
-    # with a saved statistic (its last bit may differ from the one the backward
-    # recomputes: the forward adds the squares in another order)
+    # with the saved statistic: the backward's own recomputation gives the same
+    # fp32 value (the sum of squares is accumulated in double in every kernel, so
+    # it does not depend on how a row is split over lanes), hence identical results
     dx2, dw2 = triton_rms_norm_backward(dyd, xd, wd, rms=rms)
     torch.cuda.synchronize()
-    check_bf16("rmsnorm.dx(rms given)", dx_ref, dx2)
-    torch.testing.assert_close(dw2.cpu(), dw_ref, rtol=2e-4, atol=2e-4 * float(dw_ref.abs().max()))
+    assert torch.equal(dx2.view(torch.int16).cpu(), dx.view(torch.int16).cpu())
+    assert torch.equal(dw2.cpu(), dw.cpu())
     # 3-D input
     if M % 4 == 0:
         y3, _ = triton_rms_norm_forward(xd.view(4, M // 4, N), wd)
