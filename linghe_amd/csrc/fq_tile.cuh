@@ -58,85 +58,47 @@ __device__ __forceinline__ float max_across_rows(float v) {
   return fmaxf(as_f32(b[0]), as_f32(b[1]));
 }
 
-// Write the first `len` bytes of one transposed row from LDS (`lds_row`: 128 bytes
-// as eight 16-byte chunks, chunk k stored at position k ^ swz) to the byte address
-// `dst_row`, which may have ANY alignment (per-expert transposed rows are packed
-// back to back with a stride of count_e bytes).  Called by the 8 threads
-// ch = 0..7 that share the row.  The row is cut at the 16-byte boundaries of the
-// DESTINATION: destination chunk m holds source bytes [16m - a, 16m - a + 16),
-// a = dst_row & 15, assembled from the two source chunks around it with dword
-// selects and v_alignbyte; whole chunks leave as one 16-byte store, the (at most
-// two) ragged ends as dword / byte stores of exactly the bytes of this row.
+// 16 / 8 / 4 / 2 bytes stored at ANY byte address: gfx950 runs with unaligned
+// vector memory access enabled, so one store instruction serves whatever the
+// alignment (per-expert transposed rows are packed back to back with a stride of
+// count_e bytes and start anywhere)
+struct __attribute__((packed, aligned(1))) Bytes16 { uint32_t x, y, z, w; };
+struct __attribute__((packed, aligned(1))) Bytes8 { uint32_t x, y; };
+struct __attribute__((packed, aligned(1))) Bytes4 { uint32_t x; };
+struct __attribute__((packed, aligned(1))) Bytes2 { uint16_t x; };
+__device__ __forceinline__ void store16_any(uint8_t* dst, const uint4& v) { *(Bytes16*)dst = Bytes16{v.x, v.y, v.z, v.w}; }
+
 // dword k (k = 0..3, lane-variable) of a 16-byte chunk held in four registers
-__device__ __forceinline__ uint32_t pick_dword(uint32_t o0, uint32_t o1, uint32_t o2, uint32_t o3, int k) {
-  const uint32_t lo = (k & 1) ? o1 : o0;
-  const uint32_t hi = (k & 1) ? o3 : o2;
+__device__ __forceinline__ uint32_t pick_dword(const uint4& v, int k) {
+  const uint32_t lo = (k & 1) ? v.y : v.x;
+  const uint32_t hi = (k & 1) ? v.w : v.z;
   return (k & 2) ? hi : lo;
 }
 
-// Store destination bytes [j0, j1) of the 16-byte aligned chunk at dst.
-// A ragged head (j1 == 16) or tail (j0 == 0) leaves as at most one byte, one
-// short, one dword and one qword store, each naturally aligned; a chunk ragged at
-// both ends (a row shorter than 16 bytes) goes byte by byte.
-__device__ __forceinline__ void store_t_partial(uint8_t* dst, uint32_t o0, uint32_t o1, uint32_t o2, uint32_t o3,
-                                                int j0, int j1) {
-  if (j1 == 16) {  // head: valid bytes j0..15
-    int p = j0;
-    if (p & 1) { dst[p] = (uint8_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); p += 1; }
-    if (p & 2) { *(uint16_t*)(dst + p) = (uint16_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); p += 2; }
-    if (p & 4) { *(uint32_t*)(dst + p) = pick_dword(o0, o1, o2, o3, p >> 2); p += 4; }
-    if (p & 8) { *(uint2*)(dst + 8) = make_uint2(o2, o3); }
-  } else if (j0 == 0) {  // tail: valid bytes 0..j1-1
-    int p = 0;
-    if (j1 & 8) { *(uint2*)dst = make_uint2(o0, o1); p = 8; }
-    if (j1 & 4) { *(uint32_t*)(dst + p) = pick_dword(o0, o1, o2, o3, p >> 2); p += 4; }
-    if (j1 & 2) { *(uint16_t*)(dst + p) = (uint16_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); p += 2; }
-    if (j1 & 1) { dst[p] = (uint8_t)(pick_dword(o0, o1, o2, o3, p >> 2) >> (8 * (p & 3))); }
-  } else {
-    for (int j = j0; j < j1; ++j) dst[j] = (uint8_t)(pick_dword(o0, o1, o2, o3, j >> 2) >> (8 * (j & 3)));
-  }
-}
-
-__device__ __forceinline__ void store_t_chunk(const uint8_t* lds_row, int swz, uint8_t* dst0, int a, int len, int m) {
-  const int s0 = 16 * m - a;  // source index of destination byte 0 of this chunk
-  if (s0 >= len) return;
-  uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
-  if (m >= 1) lo = *(const uint4*)(lds_row + (((m - 1) ^ swz) * 16));
-  if (m <= 7) hi = *(const uint4*)(lds_row + ((m ^ swz) * 16));
-  // window bytes 0..31 = source bytes 16(m-1) .. 16(m+1); destination byte j = window byte 16 - a + j
-  const int sb = 16 - a;  // 1..16
-  const bool b0 = (sb >> 2) & 1, b1 = (sb >> 3) & 1;
-  const uint32_t u0 = b0 ? lo.y : lo.x, u1 = b0 ? lo.z : lo.y, u2 = b0 ? lo.w : lo.z, u3 = b0 ? hi.x : lo.w;
-  const uint32_t u4 = b0 ? hi.y : hi.x, u5 = b0 ? hi.z : hi.y, u6 = b0 ? hi.w : hi.z;
-  const uint32_t t0 = b1 ? u2 : u0, t1 = b1 ? u3 : u1, t2 = b1 ? u4 : u2, t3 = b1 ? u5 : u3, t4 = b1 ? u6 : u4;
-  const uint32_t rs = (uint32_t)(sb & 3);
-  const bool al = a == 0;
-  const uint32_t o0 = al ? hi.x : __builtin_amdgcn_alignbyte(t1, t0, rs);
-  const uint32_t o1 = al ? hi.y : __builtin_amdgcn_alignbyte(t2, t1, rs);
-  const uint32_t o2 = al ? hi.z : __builtin_amdgcn_alignbyte(t3, t2, rs);
-  const uint32_t o3 = al ? hi.w : __builtin_amdgcn_alignbyte(t4, t3, rs);
-  const int j0 = s0 < 0 ? -s0 : 0;                   // first valid destination byte
-  const int j1 = (len - s0) < 16 ? (len - s0) : 16;  // one past the last valid one
-  uint8_t* dst = dst0 + 16 * m;
-  if (j0 == 0 && j1 == 16) {
-    *(uint4*)dst = make_uint4(o0, o1, o2, o3);
-  } else {
-    store_t_partial(dst, o0, o1, o2, o3, j0, j1);
-  }
-}
-
+// Write the first `len` bytes of one transposed row from LDS (`lds_row`: 128 bytes
+// as eight 16-byte chunks, chunk k stored at position k ^ swz) to `dst_row`.
+// Called by the 8 threads ch = 0..7 that share the row: thread ch owns source
+// bytes [16 ch, 16 ch + 16); a chunk cut by the end of the row leaves as at most
+// one 8-, 4-, 2- and 1-byte store.
 __device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uint8_t* dst_row, int len, int ch) {
-  const int a = (int)((uintptr_t)dst_row & 15u);
-  uint8_t* dst0 = dst_row - a;
-  store_t_chunk(lds_row, swz, dst0, a, len, ch);
-  // a ninth destination chunk exists when a misaligned row runs past 8 * 16 bytes
-  if (ch == 0 && a + len > 128) store_t_chunk(lds_row, swz, dst0, a, len, 8);
+  const int rem = len - 16 * ch;
+  if (rem <= 0) return;
+  const uint4 v = *(const uint4*)(lds_row + ((ch ^ swz) * 16));
+  uint8_t* dst = dst_row + 16 * ch;
+  if (rem >= 16) {
+    store16_any(dst, v);
+    return;
+  }
+  int p = 0;
+  if (rem & 8) { *(Bytes8*)dst = Bytes8{v.x, v.y}; p = 8; }
+  if (rem & 4) { *(Bytes4*)(dst + p) = Bytes4{pick_dword(v, p >> 2)}; p += 4; }
+  if (rem & 2) { *(Bytes2*)(dst + p) = Bytes2{(uint16_t)(pick_dword(v, p >> 2) >> (8 * (p & 3)))}; p += 2; }
+  if (rem & 1) dst[p] = (uint8_t)(pick_dword(v, p >> 2) >> (8 * (p & 3)));
 }
 
 // Quantise the tile held in registers (v[s][j] = element (rg*RPT+s, cg*8+j);
 // rows >= rows_valid must hold 0).  All threads of the workgroup must call it.
-// FULL: the tile has all 128 rows and its transposed rows are 16-byte aligned,
-// so no store needs a mask.
+// FULL: the tile has all 128 rows, so no load or store needs a mask.
 template <int KIND, bool ROUND, int MODE, int RPT, bool FULL, bool EXACT_DIV = true>
 __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], const TileOut& o,
                                                    TileShared<RPT>& sh) {
@@ -254,7 +216,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       const int c = (tid >> 3) + k * kRowsPerPass;
       if constexpr (FULL) {
         const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
-        *(uint4*)(o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16) = val;
+        store16_any(o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16, val);
       } else {
         store_t_row(sh.t + c * kGroup, (c >> 3) & 7, o.qt + o.t_off + (int64_t)c * o.t_ld, o.rows_valid, ch);
       }
@@ -267,8 +229,7 @@ template <int KIND, bool ROUND, int MODE, int RPT, bool EXACT_DIV = true>
 __device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o,
                                               TileShared<RPT>& sh) {
   // workgroup-uniform choice of the mask-free path
-  bool full = o.rows_valid == kGroup;
-  if constexpr (MODE != 0) full = full && ((((uintptr_t)(o.qt + o.t_off)) | (uintptr_t)o.t_ld) & 15) == 0;
+  const bool full = o.rows_valid == kGroup;
   if (full) quantize_tile_impl<KIND, ROUND, MODE, RPT, true, EXACT_DIV>(v, o, sh);
   else quantize_tile_impl<KIND, ROUND, MODE, RPT, false, EXACT_DIV>(v, o, sh);
 }
