@@ -35,8 +35,10 @@ int check_common(const char* fn, int64_t M, int64_t width, int round_scale, int 
   FQ_REQUIRE(M >= 0, FQ_ERR_SHAPE, "%s: negative row count", fn);
   FQ_REQUIRE(width > 0 && width % 128 == 0, FQ_ERR_SHAPE, "%s: width %lld is not a positive multiple of 128", fn,
              (long long)width);
-  FQ_REQUIRE(width <= (1 << 24), FQ_ERR_SHAPE, "%s: width too large", fn);
-  FQ_REQUIRE(M <= ((int64_t)1 << 31) - 256, FQ_ERR_SHAPE, "%s: too many rows", fn);
+  // lane offsets inside a tile are 32-bit: 128 rows of the widest input (2 * width bf16) and 128
+  // transposed rows of M bytes must stay below 4 GB
+  FQ_REQUIRE(width <= (1 << 22), FQ_ERR_SHAPE, "%s: width too large", fn);
+  FQ_REQUIRE(M <= ((int64_t)1 << 24), FQ_ERR_SHAPE, "%s: too many rows", fn);
   FQ_REQUIRE(round_scale == 0 || round_scale == 1, FQ_ERR_ARG, "%s: round_scale must be 0 or 1", fn);
   FQ_REQUIRE(fp8_kind == FQ_E4M3 || fp8_kind == FQ_E5M2, FQ_ERR_ARG, "%s: unknown fp8_kind %d", fn, fp8_kind);
   return FQ_OK;

@@ -22,6 +22,15 @@ template <> struct Fp8Traits<kE5M2Max448> { static constexpr float kMax = 448.0f
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
 
+// a value every lane of the workgroup holds identically, moved to scalar registers
+// so that addresses built from it use a scalar base and 32-bit lane offsets
+__device__ __forceinline__ int uniform32(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 // two bf16 packed in a dword -> fp32 (exact)
 __device__ __forceinline__ float bf16_lo(uint32_t p) { return as_f32(p << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t p) { return as_f32(p & 0xffff0000u); }
@@ -98,6 +107,13 @@ __device__ __forceinline__ float div_exact(float v, const Divisor& d) {
   float q0 = v * d.r;
   float e = __builtin_fmaf(-q0, d.s, v);
   return __builtin_fmaf(e, d.r, q0);
+}
+// POW2: the scale is a power of two, its reciprocal is exact and so is the
+// product v * (1/s): one multiplication IS the division
+template <bool POW2>
+__device__ __forceinline__ float div_by_scale(float v, const Divisor& d) {
+  if constexpr (POW2) return v * d.r;
+  else return div_exact(v, d);
 }
 
 // exp2(ceil(log2(s))) as torch evaluates it in fp32 (linghe/tools/util.py:61-62):

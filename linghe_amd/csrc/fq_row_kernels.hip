@@ -155,7 +155,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
         const Divisor d = make_divisor(sc);
         float qv[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) qv[j] = div_exact(y[j], d);
+        for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(y[j], d);
         uint2 pk;
         pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
         pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __rest
     const Divisor d = make_divisor(sc);
     float qv[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) qv[j] = div_exact(a[j], d);
+    for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(a[j], d);
     uint2 pk;
     pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
     pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);

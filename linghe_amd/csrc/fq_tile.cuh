@@ -99,7 +99,7 @@ __device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uin
 // Quantise the tile held in registers (v[s][j] = element (rg*RPT+s, cg*8+j);
 // rows >= rows_valid must hold 0).  All threads of the workgroup must call it.
 // FULL: the tile has all 128 rows, so no load or store needs a mask.
-template <int KIND, bool ROUND, int MODE, int RPT, bool FULL, bool EXACT_DIV = true>
+template <int KIND, bool ROUND, int MODE, int RPT, bool FULL>
 __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], const TileOut& o,
                                                    TileShared<RPT>& sh) {
   using Shape = TileShape<RPT>;
@@ -129,7 +129,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       const Divisor d = make_divisor(sc);
       const int i = rg * RPT + cg;
       sh.rdiv[i] = make_float2(d.s, d.r);
-      if (FULL || i < o.rows_valid) o.s[o.s_off + i] = sc;  // a wave writes 4*RPT consecutive floats
+      if (FULL || i < o.rows_valid) (o.s + o.s_off)[(uint32_t)i] = sc;  // a wave writes 4*RPT consecutive floats
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -142,12 +142,13 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       d.r = sr.y;
       float qv[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) qv[j] = EXACT_DIV ? div_exact(v[s][j], d) : v[s][j] * d.r;
+      for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(v[s][j], d);
       uint2 pk;
       pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
       pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
       const int i = rg * RPT + s;
-      if (FULL || i < o.rows_valid) *(uint2*)(o.q + o.q_off + (int64_t)i * o.q_ld + cg * 8) = pk;
+      // scalar tile base + 32-bit lane offset (128 rows of at most 16 KB)
+      if (FULL || i < o.rows_valid) *(uint2*)((o.q + o.q_off) + ((uint32_t)i * (uint32_t)o.q_ld + (uint32_t)cg * 8u)) = pk;
     }
   }
 
@@ -174,7 +175,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       const float sc = make_scale<KIND, ROUND>(m);
       const Divisor d = make_divisor(sc);
       sh.cdiv[tid] = make_float2(d.s, d.r);
-      o.st[o.st_off + tid] = sc;
+      (o.st + o.st_off)[(uint32_t)tid] = sc;
     }
     __syncthreads();
     Divisor cd[8];
@@ -196,7 +197,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       const Divisor d = cd[j];
       float qv[RPT];
 #pragma unroll
-      for (int s = 0; s < RPT; ++s) qv[s] = EXACT_DIV ? div_exact(v[s][j], d) : v[s][j] * d.r;
+      for (int s = 0; s < RPT; ++s) qv[s] = div_by_scale<ROUND>(v[s][j], d);
       uint8_t* p = base + (cg * 8 + j) * kGroup;
       if constexpr (RPT == 8) {
         uint2 pk;
@@ -216,22 +217,23 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       const int c = (tid >> 3) + k * kRowsPerPass;
       if constexpr (FULL) {
         const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
-        store16_any(o.qt + o.t_off + (int64_t)c * o.t_ld + ch * 16, val);
+        // scalar tile base + 32-bit lane offset (128 transposed rows of at most 2^24 bytes)
+        store16_any((o.qt + o.t_off) + ((uint32_t)c * (uint32_t)o.t_ld + (uint32_t)ch * 16u), val);
       } else {
-        store_t_row(sh.t + c * kGroup, (c >> 3) & 7, o.qt + o.t_off + (int64_t)c * o.t_ld, o.rows_valid, ch);
+        store_t_row(sh.t + c * kGroup, (c >> 3) & 7, (o.qt + o.t_off) + (uint32_t)c * (uint32_t)o.t_ld, o.rows_valid, ch);
       }
     }
     __syncthreads();  // LDS is reused by a following call
   }
 }
 
-template <int KIND, bool ROUND, int MODE, int RPT, bool EXACT_DIV = true>
+template <int KIND, bool ROUND, int MODE, int RPT>
 __device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o,
                                               TileShared<RPT>& sh) {
   // workgroup-uniform choice of the mask-free path
   const bool full = o.rows_valid == kGroup;
-  if (full) quantize_tile_impl<KIND, ROUND, MODE, RPT, true, EXACT_DIV>(v, o, sh);
-  else quantize_tile_impl<KIND, ROUND, MODE, RPT, false, EXACT_DIV>(v, o, sh);
+  if (full) quantize_tile_impl<KIND, ROUND, MODE, RPT, true>(v, o, sh);
+  else quantize_tile_impl<KIND, ROUND, MODE, RPT, false>(v, o, sh);
 }
 
 // ---------------------------------------------------------------------------

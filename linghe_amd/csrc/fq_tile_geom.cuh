@@ -45,15 +45,18 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
     g.valid = left > 0;
   } else {
     const ExpertTile et = find_expert_tile<THREADS>(b.counts, b.counts_i64, b.n_experts, rbk, scan);
-    g.valid = et.expert >= 0;
-    const int left = et.count - et.rb * kGroup;
+    // the lookup's answer is the same in every lane: keep it in scalar registers
+    const int expert = uniform32(et.expert), count = uniform32(et.count), rb = uniform32(et.rb);
+    const int64_t row_start = uniform64(et.row_start), tblock_start = uniform64(et.tblock_start);
+    g.valid = expert >= 0;
+    const int left = count - rb * kGroup;
     g.rows_valid = left < kGroup ? left : kGroup;
-    g.row0 = et.row_start + (int64_t)et.rb * kGroup;
-    g.s_base = et.row_start * (out_w / kGroup) + (int64_t)et.rb * kGroup;
-    g.s_stride = et.count;
-    g.t_base = et.row_start * out_w + (int64_t)et.rb * kGroup;
-    g.t_stride = et.count;
-    g.st_row = et.tblock_start + et.rb;
+    g.row0 = row_start + (int64_t)rb * kGroup;
+    g.s_base = row_start * (out_w / kGroup) + (int64_t)rb * kGroup;
+    g.s_stride = count;
+    g.t_base = row_start * out_w + (int64_t)rb * kGroup;
+    g.t_stride = count;
+    g.st_row = tblock_start + rb;
     if (g.row0 + g.rows_valid > M) g.valid = false;  // counts disagree with the matrix: write nothing
   }
   return g;
@@ -88,15 +91,19 @@ template <int RPT>
 __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
-  const uint16_t* p = base + (int64_t)(rg * RPT) * ld + cg * 8;
+  // base is the same for the whole workgroup (scalar registers); a tile spans at
+  // most 128 rows of at most 32 KB, so lane offsets fit 32 bits
+  const uint8_t* b = (const uint8_t*)base;
+  const uint32_t pitch = (uint32_t)ld * 2u;
+  const uint32_t off0 = (uint32_t)(rg * RPT) * pitch + (uint32_t)cg * 16u;
   if (rows_valid == kGroup) {  // workgroup-uniform: no per-row masks
 #pragma unroll
-    for (int s = 0; s < RPT; ++s) raw[s] = *(const uint4*)(p + (int64_t)s * ld);
+    for (int s = 0; s < RPT; ++s) raw[s] = *(const uint4*)(b + (off0 + (uint32_t)s * pitch));
   } else {
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
       raw[s] = make_uint4(0, 0, 0, 0);
-      if (rg * RPT + s < rows_valid) raw[s] = *(const uint4*)(p + (int64_t)s * ld);
+      if (rg * RPT + s < rows_valid) raw[s] = *(const uint4*)(b + (off0 + (uint32_t)s * pitch));
     }
   }
 }
