@@ -253,6 +253,39 @@ def build_cases(names, dev):
 
     add("cfg5a", build=rms_bwd_case)
 
+    # ---------------------------------------------------------------- next row: gather + pad + quant
+    def permute_case():
+        d = configs.next_permute_pad_quant()
+        x_cpu, probs_cpu, counts, idx_cpu = d["x"], d["probs"], d["counts"], d["indices"]
+        m, N = x_cpu.shape
+        M = idx_cpu.numel()
+        E = len(counts)
+        blocks = sum((c + 127) // 128 for c in counts)
+        cnt = torch.tensor(counts, dtype=torch.int32, device=dev)
+        idx = idx_cpu.to(dev)
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), probs=probs_cpu.to(dev), q=torch.empty((M, N), device=dev, dtype=FP8),
+                     s=torch.empty((M, N // 128), device=dev, dtype=torch.float32),
+                     qt=torch.empty((M, N), device=dev, dtype=FP8),
+                     st=torch.empty((blocks, N), device=dev, dtype=torch.float32),
+                     p=torch.empty((M,), device=dev, dtype=torch.float32))
+            s["args"] = (_p(s["x"]), _p(cnt), 0, E, blocks, _p(idx), _p(s["probs"]), 0, _p(s["p"]), _p(s["q"]),
+                         _p(s["s"]), _p(s["qt"]), _p(s["st"]), m, M, N, 0, _lib.FQ_E4M3, stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_batched_pad_permute_quant(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.batch_block_pad_permute_with_indices(x_cpu, d["indices_unpadded"], probs_cpu, counts, False)
+
+        return Case("next_permute", "triton_batch_block_pad_permute_with_indices", [M, N],
+                    configs.bytes_permute_pad_quant(N, counts), make_set, launch, cpu_fn)
+
+    add("next_permute", build=permute_case)
+
     # ---------------------------------------------------------------- plain copy of known size
     # (calibration of the FETCH_SIZE / WRITE_SIZE counters: reads and writes 256 MiB)
     def copy_case():
@@ -312,7 +345,7 @@ def time_cpu(case, budget_s):
 # the difference is the second read of x.
 CFG1_MEASURED_TRAFFIC_BYTES = 102.48e6
 
-ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c"]
+ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c", "next_permute"]
 
 
 def main():

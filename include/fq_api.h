@@ -61,6 +61,20 @@ int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_
                                int64_t total_blocks, void* q, float* s, void* qt, float* st, int64_t M,
                                int64_t N, int round_scale, int fp8_kind, void* stream);
 
+/* triton_batch_block_pad_permute_with_indices, linghe/utils/gather.py:960-1113
+ * (kernel :840-957).  x bf16 [src_rows, N]; indices int32 [M], M = sum of the
+ * counts each rounded up to 16: expert e's region of the outputs starts at the
+ * sum of the rounded counts before it, holds x[indices[start + i]] for
+ * i < count_e and zero rows up to its rounded count pc_e, and is laid out as
+ * q[(start+i)*N + c], s[start*nb + b*pc_e + i], qt[start*N + c*pc_e + i],
+ * st[(tb + i/128)*N + c].  probs (fp32 or bf16 [src_rows, n_experts], may be
+ * NULL together with prob_out): prob_out[start + i] = probs[row, e], 0 in the
+ * padding.  Indices outside [0, src_rows) read as zero rows. */
+int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
+                                 int64_t total_blocks, const void* indices, const void* probs, int probs_is_bf16,
+                                 void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
+                                 int64_t M, int64_t N, int round_scale, int fp8_kind, void* stream);
+
 /* triton_group_quant, linghe/quant/group.py:40-63.  s is [M, N/128] row-major. */
 int fq_group_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
                    void* stream);

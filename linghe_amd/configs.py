@@ -88,6 +88,24 @@ def cfg5_rmsnorm_large(M: int = 16384, n: int = 7168):
     return dict(x=x, gamma=gamma, dy=dy, eps=1e-6)
 
 
+def next_permute_pad_quant(tokens: int = 16384, n: int = 2048, n_experts: int = 32, topk: int = 2):
+    """Gather + pad-to-16 + quant (the step before the expert GEMM; shape of the
+    reference's own test, tests/test_gather.py:597): tokens*topk routed rows over
+    n_experts experts, Zipf counts with two empty experts, each expert's tokens a
+    random subset of the source rows."""
+    counts = zipf_counts(tokens * topk, n_experts, seed=1101, n_empty=2)
+    g = _gen(1101)
+    x = torch.randn(tokens, n, generator=g).to(torch.bfloat16)
+    probs = torch.rand(tokens, n_experts, generator=g)
+    parts, plain = [], []
+    for c in counts:
+        pc = (c + 15) // 16 * 16
+        src = torch.randint(0, tokens, (c,), generator=g, dtype=torch.int32)
+        plain.append(src)
+        parts += [src, torch.zeros(pc - c, dtype=torch.int32)]
+    return dict(x=x, probs=probs, counts=counts, indices=torch.cat(parts), indices_unpadded=torch.cat(plain))
+
+
 # algorithmic HBM bytes per call (each input read once, each output written once)
 def bytes_rmsnorm_quant(M, n, mode=2):
     x = 2 * M * n
@@ -122,3 +140,11 @@ def bytes_batched_swiglu_bwd(M, n, counts):
 
 def bytes_rmsnorm_bwd(M, n):
     return 2 * (2 * M * n) + 2 * M * n + 2 * n + 4 * n
+
+
+def bytes_permute_pad_quant(n, counts):
+    """each routed row read once (2 B/element) with its index and prob, both code layouts and scales written"""
+    routed = sum(counts)
+    padded = sum((c + 15) // 16 * 16 for c in counts)
+    blocks = sum((c + 127) // 128 for c in counts)
+    return 2 * routed * n + 4 * padded + 4 * routed + 2 * padded * n + 4 * padded * (n // 128) + 4 * blocks * n + 4 * padded

@@ -97,6 +97,31 @@ int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_
                       fn);
 }
 
+int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
+                                 int64_t total_blocks, const void* indices, const void* probs, int probs_is_bf16,
+                                 void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
+                                 int64_t M, int64_t N, int round_scale, int fp8_kind, void* stream) {
+  const char* fn = "fq_batched_pad_permute_quant";
+  int rc = check_common(fn, M, N, round_scale, fp8_kind);
+  if (rc) return rc;
+  if (M == 0) return FQ_OK;  // nothing routed: there is nothing to write (and empty outputs may be NULL)
+  if ((rc = check_mode_ptrs(fn, 2, q, s, qt, st))) return rc;
+  FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0 && src_rows >= 0, FQ_ERR_SHAPE, "%s: negative count", fn);
+  FQ_REQUIRE(src_rows <= ((int64_t)1 << 31) - 1, FQ_ERR_SHAPE, "%s: too many source rows for int32 indices", fn);
+  FQ_REQUIRE(M % 16 == 0, FQ_ERR_SHAPE, "%s: M (%lld) must be the sum of the counts each rounded up to 16", fn,
+             (long long)M);
+  FQ_REQUIRE((probs == nullptr) == (prob_out == nullptr), FQ_ERR_ARG, "%s: probs and prob_out go together", fn);
+  if (M == 0 || total_blocks == 0 || src_rows == 0) return FQ_OK;
+  FQ_REQUIRE(x && aligned16(x) && counts && indices && aligned16(indices), FQ_ERR_ARG,
+             "%s: x/counts/indices NULL or misaligned", fn);
+  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
+  if ((rc = check_tiles(fn, total_blocks * (N / 128)))) return rc;
+  return check_launch(fq::launch_pad_permute_quant(x, indices, probs, probs_is_bf16 != 0, prob_out, q, s, qt, st,
+                                                   src_rows, M, (int)N, round_scale, fp8_kind, counts,
+                                                   counts_is_i64 != 0, n_experts, total_blocks, (hipStream_t)stream),
+                      fn);
+}
+
 int fq_group_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
                    void* stream) {
   const char* fn = "fq_group_quant";

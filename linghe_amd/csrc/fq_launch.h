@@ -11,6 +11,11 @@ hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, fl
                                   int round_scale, int mode, int kind, const void* counts, int counts_i64,
                                   int n_experts, int64_t row_blocks, hipStream_t stream);
 
+hipError_t launch_pad_permute_quant(const void* x, const void* indices, const void* probs, int probs_bf16,
+                                    void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
+                                    int64_t M, int N, int round_scale, int kind, const void* counts, int counts_i64,
+                                    int n_experts, int64_t row_blocks, hipStream_t stream);
+
 hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_bf16, void* q, float* s, void* qt,
                                  float* st, int64_t M, int n, int round_scale, int mode, int kind,
                                  const void* counts, int counts_i64, int n_experts, int64_t row_blocks,

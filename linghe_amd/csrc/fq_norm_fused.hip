@@ -134,11 +134,13 @@ __global__ __launch_bounds__(256, 4) void rmsnorm_quant_fused_kernel(const uint1
   g.row0 = row0;
   const int64_t left = M - row0;
   g.rows_valid = left < kGroup ? (int)left : kGroup;
+  g.rows_store = g.rows_valid;
   g.s_base = row0;
   g.s_stride = M;
   g.t_base = row0;
   g.t_stride = M;
   g.st_row = slab;
+  g.expert = 0;
 
   if (tid == 0) fs.gave_up = 0;
   uint4 raw[RPT];

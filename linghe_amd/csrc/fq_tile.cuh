@@ -242,8 +242,9 @@ __device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const Ti
 struct ExpertTile {
   int expert;
   int count;            // rows of this expert
+  int pcount;           // rows of its region in the outputs: count rounded up to a multiple of `pad`
   int rb;               // 128-row block inside the expert
-  int64_t row_start;    // first global row of the expert
+  int64_t row_start;    // first global row of the expert's region (sum of the pcount before it)
   int64_t tblock_start; // sum over previous experts of ceil(count/128)
 };
 
@@ -274,9 +275,12 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
 // counts by a workgroup-wide prefix scan, THREADS experts per step; every thread
 // returns the same answer.  An out-of-range blk (host and device counts
 // disagree) yields expert = -1.
+// pad > 1: every expert's region starts at a multiple of pad rows (the reference's
+// permute-and-pad layout, pad = 16); 128 is a multiple of pad, so the number of
+// 128-row blocks of an expert does not change.
 template <int THREADS>
 __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int is_i64, int n_experts,
-                                                       int blk, ExpertScanShared& sh) {
+                                                       int blk, ExpertScanShared& sh, int pad = 1) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -286,8 +290,9 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
   for (int base = 0; base < n_experts; base += THREADS) {
     const int e = base + tid;
     const int c = (e < n_experts) ? load_count(counts, is_i64, e) : 0;
+    const int pc = (c + pad - 1) / pad * pad;
     const int nb = (c + kGroup - 1) / kGroup;
-    const int rows = wave_inclusive_scan(c);
+    const int rows = wave_inclusive_scan(pc);
     const int blocks = wave_inclusive_scan(nb);
     if (base != 0) __syncthreads();  // readers of the previous step are done
     if (lane == 63) { sh.wave_rows[wave] = rows; sh.wave_blocks[wave] = blocks; }
@@ -305,8 +310,9 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
       ExpertTile t;
       t.expert = e;
       t.count = c;
+      t.pcount = pc;
       t.rb = blk - excl_blocks;
-      t.row_start = (int64_t)(rows_before + rows - c);
+      t.row_start = (int64_t)(rows_before + rows - pc);
       t.tblock_start = excl_blocks;
       sh.found = t;
     }

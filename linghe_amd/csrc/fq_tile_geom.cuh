@@ -10,11 +10,13 @@ namespace fq {
 // ---------------------------------------------------------------------------
 struct TileGeom {
   int64_t row0;      // first global row of the tile
-  int rows_valid;
+  int rows_valid;    // rows that exist in the input (and in the outputs unless padded)
+  int rows_store;    // rows written to the outputs (>= rows_valid; the extra ones hold zeros)
   int cb;            // 128-column block of the input
   int64_t s_base, s_stride;
   int64_t t_base, t_stride;
   int64_t st_row;
+  int expert;        // per-expert forms: the expert the tile belongs to
   bool valid;
 };
 
@@ -22,6 +24,7 @@ struct BatchArgs {
   const void* counts;  // device, int32 or int64, [n_experts]
   int counts_i64;
   int n_experts;
+  int pad;             // 0/1: experts packed back to back; 16: each expert's region padded to 16 rows
 };
 
 // out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
@@ -37,27 +40,34 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
     g.row0 = (int64_t)rbk * kGroup;
     const int64_t left = M - g.row0;
     g.rows_valid = left < kGroup ? (int)left : kGroup;
+    g.rows_store = g.rows_valid;
     g.s_base = g.row0;
     g.s_stride = M;
     g.t_base = g.row0;
     g.t_stride = M;
     g.st_row = rbk;
+    g.expert = 0;
     g.valid = left > 0;
   } else {
-    const ExpertTile et = find_expert_tile<THREADS>(b.counts, b.counts_i64, b.n_experts, rbk, scan);
+    const ExpertTile et = find_expert_tile<THREADS>(b.counts, b.counts_i64, b.n_experts, rbk, scan,
+                                                    b.pad > 1 ? b.pad : 1);
     // the lookup's answer is the same in every lane: keep it in scalar registers
     const int expert = uniform32(et.expert), count = uniform32(et.count), rb = uniform32(et.rb);
+    const int pcount = uniform32(et.pcount);
     const int64_t row_start = uniform64(et.row_start), tblock_start = uniform64(et.tblock_start);
     g.valid = expert >= 0;
+    g.expert = expert;
     const int left = count - rb * kGroup;
+    const int pleft = pcount - rb * kGroup;
     g.rows_valid = left < kGroup ? left : kGroup;
+    g.rows_store = pleft < kGroup ? pleft : kGroup;
     g.row0 = row_start + (int64_t)rb * kGroup;
     g.s_base = row_start * (out_w / kGroup) + (int64_t)rb * kGroup;
-    g.s_stride = count;
+    g.s_stride = pcount;
     g.t_base = row_start * out_w + (int64_t)rb * kGroup;
-    g.t_stride = count;
+    g.t_stride = pcount;
     g.st_row = tblock_start + rb;
-    if (g.row0 + g.rows_valid > M) g.valid = false;  // counts disagree with the matrix: write nothing
+    if (g.row0 + g.rows_store > M) g.valid = false;  // counts disagree with the matrix: write nothing
   }
   return g;
 }
@@ -82,7 +92,7 @@ __device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g,
   o.t_ld = g.t_stride;
   o.st = p.st;
   o.st_off = g.st_row * out_w + (int64_t)ocb * kGroup;
-  o.rows_valid = g.rows_valid;
+  o.rows_valid = g.rows_store;
   return o;
 }
 

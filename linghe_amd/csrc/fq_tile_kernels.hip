@@ -29,6 +29,68 @@ __global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __
 }
 
 // ---------------------------------------------------------------------------
+// gather + pad + blockwise quant (linghe/utils/gather.py:840-1113): expert e's
+// region of the outputs holds count_e gathered rows, x[indices[start_e + i]],
+// followed by zero rows up to the next multiple of 16; every per-expert layout
+// uses the padded count as its stride.  prob_out[start_e + i] = probs[row, e].
+// ---------------------------------------------------------------------------
+template <int KIND, bool ROUND>
+__global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* __restrict__ x,
+                                                                const int* __restrict__ indices,
+                                                                const void* __restrict__ probs, int probs_bf16,
+                                                                void* __restrict__ prob_out, OutPtrs out,
+                                                                int64_t src_rows, int64_t M, int N,
+                                                                BatchArgs batch) {
+  constexpr int RPT = 8;
+  __shared__ TileShared<RPT> sh;
+  __shared__ ExpertScanShared scan;
+  const TileGeom g = resolve_tile<true, 256>(M, N / kGroup, N, batch, scan);
+  if (!g.valid) return;
+  const int cg = threadIdx.x & 15;
+  const int rg = threadIdx.x >> 4;
+  // the 8 source rows of this thread: two 16-byte loads (regions start at multiples of 16 rows)
+  int src[RPT];
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) src[s] = -1;
+  if (g.row0 + rg * RPT < M) {  // M is a multiple of 16: the eight entries exist together
+    const int4* ip = (const int4*)(indices + g.row0 + rg * RPT);
+    const int4 a = ip[0], b = ip[1];
+    src[0] = a.x; src[1] = a.y; src[2] = a.z; src[3] = a.w;
+    src[4] = b.x; src[5] = b.y; src[6] = b.z; src[7] = b.w;
+  }
+  uint4 raw[RPT];
+  const uint16_t* col = x + (int64_t)g.cb * kGroup + cg * 8;
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) {
+    raw[s] = make_uint4(0, 0, 0, 0);
+    // rows of the padding, and indices that do not name a source row, read as zero
+    if (rg * RPT + s < g.rows_valid && (uint32_t)src[s] < (uint64_t)src_rows)
+      raw[s] = *(const uint4*)(col + (int64_t)src[s] * N);
+  }
+  if (probs != nullptr && g.cb == 0 && threadIdx.x < kGroup) {
+    const int i = threadIdx.x;
+    if (i < g.rows_store) {
+      const int e = g.expert;
+      float pv = 0.f;
+      const int r = indices[g.row0 + i];
+      const bool live = i < g.rows_valid && (uint32_t)r < (uint64_t)src_rows;
+      const int64_t at = (int64_t)r * batch.n_experts + e;
+      if (probs_bf16) {
+        uint16_t h = live ? ((const uint16_t*)probs)[at] : (uint16_t)0;
+        ((uint16_t*)prob_out)[g.row0 + i] = h;
+      } else {
+        if (live) pv = ((const float*)probs)[at];
+        ((float*)prob_out)[g.row0 + i] = pv;
+      }
+    }
+  }
+  float v[RPT][8];
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
+  quantize_tile<KIND, ROUND, 2, RPT>(v, make_out(out, g, N, g.cb), sh);
+}
+
+// ---------------------------------------------------------------------------
 // SwiGLU forward + quant.  y = (sigmoid(x1)*x1)*x2 [*w_row]   (fp32)
 // ---------------------------------------------------------------------------
 struct RowWeight {
@@ -202,6 +264,22 @@ hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, fl
         FQ_DISPATCH_BOOL(batched, B,
           hipLaunchKernelGGL((blockwise_quant_kernel<K, R, MD, B>), grid, block, 0, stream,
                              (const uint16_t*)x, out, M, N, b);))))
+  return hipGetLastError();
+}
+
+hipError_t launch_pad_permute_quant(const void* x, const void* indices, const void* probs, int probs_bf16,
+                                    void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
+                                    int64_t M, int N, int round_scale, int kind, const void* counts, int counts_i64,
+                                    int n_experts, int64_t row_blocks, hipStream_t stream) {
+  OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
+  BatchArgs b{counts, counts_i64, n_experts, 16};
+  const int64_t tiles = row_blocks * (N / kGroup);
+  if (tiles == 0) return hipSuccess;
+  const dim3 grid((unsigned)tiles), block(256);
+  FQ_DISPATCH_KIND(kind, K,
+    FQ_DISPATCH_BOOL(round_scale, R,
+      hipLaunchKernelGGL((pad_permute_quant_kernel<K, R>), grid, block, 0, stream, (const uint16_t*)x,
+                         (const int*)indices, probs, probs_bf16, prob_out, out, src_rows, M, N, b);))
   return hipGetLastError();
 }
 

@@ -22,6 +22,9 @@ reference holds no golden vectors for this path):
   (gradcheck) and against torch.nn.RMSNorm; a dropped 1/n, a wrong power of r
   or a transposed operand fails them.
 * ``swiglu_*`` - closed-form derivatives checked against fp64 autograd.
+* ``batch_block_pad_permute_with_indices`` / ``pad_indices`` - element-by-element
+  loops over the kernel's published offsets (padded expert starts, padded
+  strides, zero padding rows with the floor scale) on a tiny ragged case.
 * e5m2 variants - parity unpinned by the reference (it has no e5m2 path);
   pinned only by the same software encoder and invariants.
 """
@@ -237,6 +240,53 @@ def _as_count_list(counts):
 def batch_blockwise_quant(xs, counts, round_scale: bool = False, fp8_dtype=E4M3):
     """tests/test_blockwise_quant.py:17-43."""
     return _pack_experts(xs.float(), _as_count_list(counts), round_scale, fp8_dtype)
+
+
+def pad_indices(indices, counts, multiple: int = 16):
+    """The index layout the gather kernel reads (linghe/utils/gather.py:871-875):
+    expert e's entries start at the sum of the counts before it, each rounded up
+    to `multiple`; the padding entries are zero and never used."""
+    counts = _as_count_list(counts)
+    out, s = [], 0
+    for c in counts:
+        pc = (c + multiple - 1) // multiple * multiple
+        out.append(indices[s:s + c].to(torch.int32))
+        out.append(torch.zeros(pc - c, dtype=torch.int32))
+        s += c
+    return torch.cat(out) if out else torch.zeros(0, dtype=torch.int32)
+
+
+def batch_block_pad_permute_with_indices(x, indices, probs, counts, round_scale: bool = True,
+                                         fp8_dtype=E4M3):
+    """tests/test_gather.py:150-197: per expert (empty ones skipped) the rows
+    x[indices[s:s+c]] in fp32, zero-padded to a multiple of 16 rows
+    (linghe/tools/util.py:69-82, padding=True), blockwise quantised; the four
+    results flattened and concatenated in expert order; probs[:, e][index]
+    zero-padded likewise.  `indices` is the UNPADDED concatenation."""
+    counts = _as_count_list(counts)
+    qs, ss, qts, sts, ps = [], [], [], [], []
+    s = 0
+    for e, c in enumerate(counts):
+        if c == 0:
+            continue
+        index = indices[s:s + c].long()
+        y = x[index].float()
+        pad = (c + 15) // 16 * 16 - c
+        if pad:
+            y = torch.nn.functional.pad(y, (0, 0, 0, pad))
+        q, sc, qt, st = blockwise_quant(y, round_scale, fp8_dtype)
+        qs.append(q.reshape(-1))
+        ss.append(sc.reshape(-1))
+        qts.append(qt.reshape(-1))
+        sts.append(st.reshape(-1))
+        if probs is not None:
+            ps.append(torch.nn.functional.pad(probs[:, e][index], (0, pad)))
+        s += c
+    if not qs:
+        z8, z32 = torch.empty((0,), dtype=fp8_dtype), torch.empty((0,), dtype=torch.float32)
+        return z8, z32, z8.clone(), z32.clone(), (z32.clone() if probs is not None else None)
+    return (torch.cat(qs), torch.cat(ss), torch.cat(qts), torch.cat(sts),
+            torch.cat(ps) if probs is not None else None)
 
 
 def batch_weighted_silu_and_block_quant_forward(xs, weight, counts,

@@ -226,6 +226,54 @@ def test_batched_layouts_elementwise(counts):
     assert float(s2[s0 * nb]) == group_amax_scale(xs.float().numpy()[s0, :128])
 
 
+def test_pad_permute_layouts_elementwise():
+    """gather + pad-to-16 + quant against the offsets the reference kernel writes
+    (linghe/utils/gather.py:871-940): region start psi = sum of padded counts,
+    strides = padded count, padding rows zero with the floor scale."""
+    g = torch.Generator().manual_seed(77)
+    counts = [5, 0, 130, 16]
+    m, N, E = 40, 256, len(counts)
+    nb = N // 128
+    x = torch.randn(m, N, generator=g).to(torch.bfloat16)
+    probs = torch.rand(m, E, generator=g)
+    idx = torch.randint(0, m, (sum(counts),), generator=g)
+    q, s, qt, st, p = O.batch_block_pad_permute_with_indices(x, idx, probs, counts, round_scale=False)
+    padded = O.pad_indices(idx, counts)
+    pcs = [(c + 15) // 16 * 16 for c in counts]
+    assert padded.numel() == sum(pcs) == q.numel() // N == p.numel()
+    qf = q.float().reshape(-1).numpy()
+    qtf = qt.float().reshape(-1).numpy()
+    sf, stf, pf = s.numpy(), st.numpy(), p.numpy()
+    xf = x.float().numpy()
+    psi = blk = src0 = 0
+    for e, (c, pc) in enumerate(zip(counts, pcs)):
+        for i in range(pc):
+            row = xf[int(idx[src0 + i])] if i < c else np.zeros(N, dtype=np.float32)
+            if i < c:
+                assert int(padded[psi + i]) == int(idx[src0 + i])
+                assert pf[psi + i] == float(probs[int(idx[src0 + i]), e])
+            else:
+                assert pf[psi + i] == 0.0
+            for b in range(nb):
+                sc = group_amax_scale(row[b * 128:(b + 1) * 128])
+                assert sf[psi * nb + b * pc + i] == sc
+                for c_ in (b * 128, b * 128 + 77):
+                    want = float(torch.tensor(row[c_] / sc).to(torch.float8_e4m3fn).float())
+                    assert qf[(psi + i) * N + c_] == want
+            # transposed copy: column c_ of the padded [pc, N] block, 128-row groups
+            rbk = i // 128
+            rows = [xf[int(idx[src0 + k])] if k < c else np.zeros(N, dtype=np.float32)
+                    for k in range(rbk * 128, min(pc, rbk * 128 + 128))]
+            for c_ in (3, 200):
+                sc = group_amax_scale([r[c_] for r in rows])
+                assert stf[(blk + rbk) * N + c_] == sc
+                want = float(torch.tensor(row[c_] / sc).to(torch.float8_e4m3fn).float())
+                assert qtf[psi * N + c_ * pc + i] == want
+        psi += pc
+        blk += (c + 127) // 128
+        src0 += c
+
+
 def test_backward_layout_halves():
     """dx1 | dx2 share one [2n/128, M] scale tensor and one [2n, M] transposed
     tensor: rows 0..nb-1 / columns 0..n-1 belong to dx1 (linghe/utils/silu.py:382-420)."""
