@@ -286,6 +286,63 @@ def build_cases(names, dev):
 
     add("next_permute", build=permute_case)
 
+    # ---------------------------------------------------------------- next rows: bf16 SwiGLU, weight block quant
+    def wsilu_case(backward):
+        M, N = 8192, 4096  # x [M, N] = gate | up
+        g = torch.Generator().manual_seed(1102)
+        x_cpu = torch.randn(M, N, generator=g).to(torch.bfloat16)
+        w_cpu = torch.rand(M, 1, generator=g)
+        dy_cpu = torch.randn(M, N // 2, generator=g).to(torch.bfloat16)
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), w=w_cpu.to(dev))
+            if backward:
+                s.update(dy=dy_cpu.to(dev), dx=torch.empty((M, N), device=dev, dtype=torch.bfloat16),
+                         dw=torch.empty((M, 1), device=dev, dtype=torch.float32))
+                s["args"] = (_p(s["dy"]), _p(s["x"]), _p(s["w"]), 0, _p(s["dx"]), _p(s["dw"]), M, N // 2, stream)
+            else:
+                s["y"] = torch.empty((M, N // 2), device=dev, dtype=torch.bfloat16)
+                s["args"] = (_p(s["x"]), _p(s["w"]), 0, _p(s["y"]), M, N // 2, stream)
+            return s
+
+        def launch(s):
+            _lib.check((L.fq_swiglu_bwd if backward else L.fq_swiglu_fwd)(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.weighted_silu_backward(dy_cpu, x_cpu, w_cpu) if backward else O.weighted_silu_forward(x_cpu, w_cpu)
+
+        nbytes = (2 * M * N + 2 * M * (N // 2) + 4 * M) + ((2 * M * N + 4 * M) if backward else 0)
+        return Case("next_wsilu_bwd" if backward else "next_wsilu_fwd",
+                    "triton_weighted_silu_backward" if backward else "triton_weighted_silu_forward", [M, N], nbytes,
+                    make_set, launch, cpu_fn)
+
+    add("next_wsilu_fwd", build=lambda: wsilu_case(False))
+    add("next_wsilu_bwd", build=lambda: wsilu_case(True))
+
+    def block_quant_case():
+        M, N = 8192, 4096
+        g = torch.Generator().manual_seed(1103)
+        x_cpu = (torch.randn(M, N, generator=g) ** 3).to(torch.bfloat16)
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), q=torch.empty((M, N), device=dev, dtype=FP8),
+                     s=torch.empty((M // 128, N // 128), device=dev, dtype=torch.float32))
+            s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), M, N, 1, _lib.FQ_E4M3, stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_block_quant(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.block_quant_128(x_cpu, True)
+
+        return Case("next_block_quant", "triton_block_quant(round_scale=True)", [M, N],
+                    3 * M * N + 4 * (M // 128) * (N // 128), make_set, launch, cpu_fn)
+
+    add("next_block_quant", build=block_quant_case)
+
     # ---------------------------------------------------------------- plain copy of known size
     # (calibration of the FETCH_SIZE / WRITE_SIZE counters: reads and writes 256 MiB)
     def copy_case():
@@ -345,7 +402,8 @@ def time_cpu(case, budget_s):
 # the difference is the second read of x.
 CFG1_MEASURED_TRAFFIC_BYTES = 102.48e6
 
-ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c", "next_permute"]
+ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c", "next_permute",
+       "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant"]
 
 
 def main():

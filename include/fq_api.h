@@ -75,6 +75,23 @@ int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_i
                                  void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
                                  int64_t M, int64_t N, int round_scale, int fp8_kind, void* stream);
 
+/* triton_block_quant, linghe/quant/block.py:32-62 (kernel :11-29): one scale per
+ * 128x128 block of a weight.  x bf16 [M,N], M and N multiples of 128;
+ * q [M,N], s [M/128, N/128]. */
+int fq_block_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
+                   void* stream);
+
+/* triton_weighted_silu_forward, linghe/utils/silu.py:98-127 (kernel :63-94).
+ * x bf16 [M, 2n] (gate | up), weight [M] fp32 or bf16 or NULL; out bf16 [M, n]. */
+int fq_swiglu_fwd(const void* x, const void* weight, int weight_is_bf16, void* out, int64_t M, int64_t n,
+                  void* stream);
+
+/* triton_weighted_silu_backward, linghe/utils/silu.py:177-210 (kernel :130-174).
+ * g bf16 [M,n], x bf16 [M,2n]; dx bf16 [M,2n] (dx1 | dx2); dw [M] in the weight's
+ * dtype, NULL together with weight. */
+int fq_swiglu_bwd(const void* g, const void* x, const void* weight, int weight_is_bf16, void* dx, void* dw,
+                  int64_t M, int64_t n, void* stream);
+
 /* triton_group_quant, linghe/quant/group.py:40-63.  s is [M, N/128] row-major. */
 int fq_group_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
                    void* stream);

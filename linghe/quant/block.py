@@ -1,1 +1,5 @@
-from linghe_amd.quant.block import triton_batch_blockwise_quant, triton_blockwise_quant  # noqa: F401
+from linghe_amd.quant.block import (  # noqa: F401
+    triton_batch_blockwise_quant,
+    triton_block_quant,
+    triton_blockwise_quant,
+)

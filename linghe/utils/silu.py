@@ -3,4 +3,6 @@ from linghe_amd.utils.silu import (  # noqa: F401
     triton_batch_weighted_silu_and_block_quant_forward,
     triton_silu_and_block_quant_backward,
     triton_silu_and_block_quant_forward,
+    triton_weighted_silu_backward,
+    triton_weighted_silu_forward,
 )

@@ -28,6 +28,9 @@ SIGNATURES = {
     "fq_blockwise_quant": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_blockwise_quant": [_P, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_pad_permute_quant": [_P, _P, _I, _I, _L, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _P],
+    "fq_block_quant": [_P, _P, _P, _L, _L, _I, _I, _P],
+    "fq_swiglu_fwd": [_P, _P, _I, _P, _L, _L, _P],
+    "fq_swiglu_bwd": [_P, _P, _P, _I, _P, _P, _L, _L, _P],
     "fq_group_quant": [_P, _P, _P, _L, _L, _I, _I, _P],
     "fq_rmsnorm_fwd": [_P, _P, _P, _P, _L, _L, _F, _I, _P],
     "fq_rmsnorm_bwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _P],

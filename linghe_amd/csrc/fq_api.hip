@@ -244,6 +244,44 @@ int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, fl
                       fn);
 }
 
+int fq_block_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
+                   void* stream) {
+  const char* fn = "fq_block_quant";
+  int rc = check_common(fn, M, N, round_scale, fp8_kind);
+  if (rc) return rc;
+  FQ_REQUIRE(M % 128 == 0, FQ_ERR_SHAPE, "%s: M (%lld) is not a multiple of 128", fn, (long long)M);
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && q && s && aligned16(x), FQ_ERR_ARG, "%s: NULL or misaligned pointer", fn);
+  FQ_REQUIRE((reinterpret_cast<uintptr_t>(q) & 7u) == 0, FQ_ERR_ARG, "%s: q must be 8-byte aligned", fn);
+  if ((rc = check_tiles(fn, (M / 128) * (N / 128)))) return rc;
+  return check_launch(fq::launch_block_quant(x, q, s, M, (int)N, round_scale, fp8_kind, (hipStream_t)stream), fn);
+}
+
+int fq_swiglu_fwd(const void* x, const void* weight, int weight_is_bf16, void* out, int64_t M, int64_t n,
+                  void* stream) {
+  const char* fn = "fq_swiglu_fwd";
+  int rc = check_common(fn, M, n, 0, FQ_E4M3);
+  if (rc) return rc;
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && out && aligned16(x) && aligned16(out), FQ_ERR_ARG, "%s: NULL or misaligned pointer", fn);
+  return check_launch(fq::launch_swiglu_rows_fwd(x, weight, weight_is_bf16 != 0, out, M, (int)n, (hipStream_t)stream),
+                      fn);
+}
+
+int fq_swiglu_bwd(const void* g, const void* x, const void* weight, int weight_is_bf16, void* dx, void* dw,
+                  int64_t M, int64_t n, void* stream) {
+  const char* fn = "fq_swiglu_bwd";
+  int rc = check_common(fn, M, n, 0, FQ_E4M3);
+  if (rc) return rc;
+  FQ_REQUIRE((weight == nullptr) == (dw == nullptr), FQ_ERR_ARG, "%s: weight and dw go together", fn);
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(g && x && dx && aligned16(g) && aligned16(x) && aligned16(dx), FQ_ERR_ARG,
+             "%s: NULL or misaligned pointer", fn);
+  return check_launch(fq::launch_swiglu_rows_bwd(g, x, weight, weight_is_bf16 != 0, dx, dw, M, (int)n,
+                                                 (hipStream_t)stream),
+                      fn);
+}
+
 int fq_swiglu_quant_fwd(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t n,
                         int round_scale, int output_mode, int fp8_kind, void* stream) {
   const char* fn = "fq_swiglu_quant_fwd";

@@ -43,6 +43,15 @@ __device__ __forceinline__ void unpack8(const uint4& p, float (&v)[8]) {
   v[6] = bf16_lo(p.w); v[7] = bf16_hi(p.w);
 }
 
+// per-row weight of the weighted SwiGLU forms: [M] fp32 or bf16, nullptr = unweighted
+struct RowWeight {
+  const void* w;
+  int is_bf16;
+};
+__device__ __forceinline__ float load_weight(const RowWeight& w, int64_t r) {
+  return w.is_bf16 ? as_f32((uint32_t)((const uint16_t*)w.w)[r] << 16) : ((const float*)w.w)[r];
+}
+
 // fp32 pair -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950)
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float floatx2_t __attribute__((ext_vector_type(2)));

@@ -49,4 +49,12 @@ hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, 
 hipError_t launch_group_quant(const void* x, void* q, float* s, int64_t n_groups, int round_scale, int kind,
                               hipStream_t stream);
 
+// bf16 SwiGLU rows (no quantisation) and the 128x128 weight block quantiser
+hipError_t launch_swiglu_rows_fwd(const void* x, const void* weight, int weight_bf16, void* out, int64_t M, int n,
+                                  hipStream_t stream);
+hipError_t launch_swiglu_rows_bwd(const void* g, const void* x, const void* weight, int weight_bf16, void* dx,
+                                  void* dw, int64_t M, int n, hipStream_t stream);
+hipError_t launch_block_quant(const void* x, void* q, float* s, int64_t M, int N, int round_scale, int kind,
+                              hipStream_t stream);
+
 }  // namespace fq

@@ -444,4 +444,198 @@ hipError_t launch_group_quant(const void* x, void* q, float* s, int64_t n_groups
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// bf16 SwiGLU without quantisation (linghe/utils/silu.py:98-210): one wave per
+// row, lanes stride over the row in 16-byte chunks, four chunks in flight.
+//   forward:  out = ((sigmoid(x1)*x1)*x2)[*w_row]                    -> bf16 [M, n]
+//   backward: dx1 = h*sg + ((h*x1)*(1-sg))*sg, dx2 = g[*w]*(sg*x1)   -> bf16 [M, 2n]
+//             dw_row = sum_c g*((sg*x1)*x2)   (weighted form only)
+// in the order fp32 autograd evaluates them (the SwiGLU + quant kernels use the
+// same expressions).
+// ---------------------------------------------------------------------------
+template <bool WEIGHTED>
+__global__ __launch_bounds__(64) void swiglu_fwd_rows_kernel(const uint16_t* __restrict__ x, RowWeight weight,
+                                                             uint16_t* __restrict__ out, int64_t M, int n) {
+  const int lane = threadIdx.x;
+  const int chunks = n >> 3;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint16_t* p = x + row * 2 * (int64_t)n;
+    float w = 1.0f;
+    if constexpr (WEIGHTED) w = load_weight(weight, row);
+    for (int c0 = 0; c0 < chunks; c0 += 256) {
+      uint4 r1[4], r2[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * 64 + lane;
+        r1[u] = make_uint4(0, 0, 0, 0);
+        r2[u] = make_uint4(0, 0, 0, 0);
+        if (c < chunks) {
+          r1[u] = *(const uint4*)(p + c * 8);
+          r2[u] = *(const uint4*)(p + n + c * 8);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * 64 + lane;
+        float a[8], b[8], y[8];
+        unpack8(r1[u], a);
+        unpack8(r2[u], b);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          y[j] = (sigmoid_f32(a[j]) * a[j]) * b[j];
+          if constexpr (WEIGHTED) y[j] = y[j] * w;
+        }
+        if (c < chunks) *(uint4*)(out + row * n + c * 8) = pack8_bf16(y);
+      }
+    }
+  }
+}
+
+template <bool WEIGHTED>
+__global__ __launch_bounds__(64) void swiglu_bwd_rows_kernel(const uint16_t* __restrict__ gr,
+                                                             const uint16_t* __restrict__ x, RowWeight weight,
+                                                             uint16_t* __restrict__ dx, void* __restrict__ dw,
+                                                             int64_t M, int n) {
+  const int lane = threadIdx.x;
+  const int chunks = n >> 3;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint16_t* p = x + row * 2 * (int64_t)n;
+    const uint16_t* gp = gr + row * (int64_t)n;
+    uint16_t* o = dx + row * 2 * (int64_t)n;
+    float w = 1.0f;
+    if constexpr (WEIGHTED) w = load_weight(weight, row);
+    float dws = 0.f;
+    for (int c0 = 0; c0 < chunks; c0 += 128) {
+      uint4 r1[2], r2[2], rg[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int c = c0 + u * 64 + lane;
+        r1[u] = make_uint4(0, 0, 0, 0);
+        r2[u] = make_uint4(0, 0, 0, 0);
+        rg[u] = make_uint4(0, 0, 0, 0);
+        if (c < chunks) {
+          r1[u] = *(const uint4*)(p + c * 8);
+          r2[u] = *(const uint4*)(p + n + c * 8);
+          rg[u] = *(const uint4*)(gp + c * 8);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int c = c0 + u * 64 + lane;
+        float a[8], b[8], go[8], d1[8], d2[8];
+        unpack8(r1[u], a);
+        unpack8(r2[u], b);
+        unpack8(rg[u], go);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float sg = sigmoid_f32(a[j]);
+          const float sx = sg * a[j];
+          float gw = go[j];
+          if constexpr (WEIGHTED) {
+            dws += go[j] * (sx * b[j]);
+            gw = go[j] * w;
+          }
+          const float h = gw * b[j];
+          d2[j] = gw * sx;
+          d1[j] = h * sg + ((h * a[j]) * (1.0f - sg)) * sg;
+        }
+        if (c < chunks) {
+          *(uint4*)(o + c * 8) = pack8_bf16(d1);
+          *(uint4*)(o + n + c * 8) = pack8_bf16(d2);
+        }
+      }
+    }
+    if constexpr (WEIGHTED) {
+      dws = wave_sum(dws);
+      if (lane == 0) {
+        if (weight.is_bf16) ((uint16_t*)dw)[row] = (uint16_t)(pack_bf16x2(dws, 0.f) & 0xffffu);
+        else ((float*)dw)[row] = dws;
+      }
+    }
+  }
+}
+
+hipError_t launch_swiglu_rows_fwd(const void* x, const void* weight, int weight_bf16, void* out, int64_t M, int n,
+                                  hipStream_t stream) {
+  if (M == 0) return hipSuccess;
+  int64_t wgs = M < 256 * 32 ? M : 256 * 32;
+  RowWeight w{weight, weight_bf16};
+  if (weight) hipLaunchKernelGGL(swiglu_fwd_rows_kernel<true>, dim3((unsigned)wgs), dim3(64), 0, stream,
+                                 (const uint16_t*)x, w, (uint16_t*)out, M, n);
+  else hipLaunchKernelGGL(swiglu_fwd_rows_kernel<false>, dim3((unsigned)wgs), dim3(64), 0, stream,
+                          (const uint16_t*)x, w, (uint16_t*)out, M, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_swiglu_rows_bwd(const void* g, const void* x, const void* weight, int weight_bf16, void* dx,
+                                  void* dw, int64_t M, int n, hipStream_t stream) {
+  if (M == 0) return hipSuccess;
+  int64_t wgs = M < 256 * 32 ? M : 256 * 32;
+  RowWeight w{weight, weight_bf16};
+  if (weight) hipLaunchKernelGGL(swiglu_bwd_rows_kernel<true>, dim3((unsigned)wgs), dim3(64), 0, stream,
+                                 (const uint16_t*)g, (const uint16_t*)x, w, (uint16_t*)dx, dw, M, n);
+  else hipLaunchKernelGGL(swiglu_bwd_rows_kernel<false>, dim3((unsigned)wgs), dim3(64), 0, stream,
+                          (const uint16_t*)g, (const uint16_t*)x, w, (uint16_t*)dx, dw, M, n);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// 128x128 block quant of a weight (linghe/quant/block.py:11-62): one scale per
+// block, s[rb * (N/128) + cb]; one workgroup per block, 8 rows x 8 columns per
+// thread as in the tile kernels, no transposed copy.
+// ---------------------------------------------------------------------------
+template <int KIND, bool ROUND>
+__global__ __launch_bounds__(256) void block_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
+                                                          float* __restrict__ s, int N) {
+  __shared__ float wmax[4];
+  const int ncb = N / kGroup;
+  const int rb = blockIdx.x / ncb, cb = blockIdx.x - rb * ncb;
+  const int cg = threadIdx.x & 15, rg = threadIdx.x >> 4;
+  const uint8_t* src = (const uint8_t*)(x + ((int64_t)rb * kGroup) * N + (int64_t)cb * kGroup);
+  uint8_t* dst = q + ((int64_t)rb * kGroup) * N + (int64_t)cb * kGroup;
+  const uint32_t off = (uint32_t)(rg * 8) * (uint32_t)N + (uint32_t)cg * 8u;  // in elements
+  uint4 raw[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) raw[k] = *(const uint4*)(src + 2u * (off + (uint32_t)k * (uint32_t)N));
+  float m = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float a[8];
+    unpack8(raw[k], a);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(a[j]));
+  }
+  m = wave_max(m);
+  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+  const float sc = make_scale<KIND, ROUND>(m);
+  const Divisor d = make_divisor(sc);
+  if (threadIdx.x == 0) s[(int64_t)rb * ncb + cb] = sc;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float a[8], qv[8];
+    unpack8(raw[k], a);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(a[j], d);
+    uint2 pk;
+    pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+    pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+    *(uint2*)(dst + (off + (uint32_t)k * (uint32_t)N)) = pk;
+  }
+}
+
+hipError_t launch_block_quant(const void* x, void* q, float* s, int64_t M, int N, int round_scale, int kind,
+                              hipStream_t stream) {
+  const int64_t blocks = (M / kGroup) * (N / kGroup);
+  if (blocks == 0) return hipSuccess;
+  const dim3 grid((unsigned)blocks), block(256);
+#define FQ_BQ(KINDV, ROUNDV) \
+  hipLaunchKernelGGL((block_quant_kernel<KINDV, ROUNDV>), grid, block, 0, stream, (const uint16_t*)x, (uint8_t*)q, s, N)
+  if (kind == kE5M2) { if (round_scale) FQ_BQ(kE5M2, true); else FQ_BQ(kE5M2, false); }
+  else { if (round_scale) FQ_BQ(kE4M3, true); else FQ_BQ(kE4M3, false); }
+#undef FQ_BQ
+  return hipGetLastError();
+}
+
 }  // namespace fq

@@ -93,14 +93,6 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
 // ---------------------------------------------------------------------------
 // SwiGLU forward + quant.  y = (sigmoid(x1)*x1)*x2 [*w_row]   (fp32)
 // ---------------------------------------------------------------------------
-struct RowWeight {
-  const void* w;   // [M] fp32 or bf16, nullptr = unweighted
-  int is_bf16;
-};
-__device__ __forceinline__ float load_weight(const RowWeight& w, int64_t r) {
-  return w.is_bf16 ? as_f32((uint32_t)((const uint16_t*)w.w)[r] << 16) : ((const float*)w.w)[r];
-}
-
 template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED>
 __global__ __launch_bounds__(256) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {

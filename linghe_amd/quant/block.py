@@ -7,6 +7,31 @@ import torch
 from .. import _lib
 
 
+def triton_block_quant(x, block_size=128, round_scale=False, *, fp8_dtype=torch.float8_e4m3fn):
+    """
+    blockwise quantize x, used for blockwise recipe for weight in megatron
+    Args:
+        x: input tensor, bf16 [M, N], M and N multiples of 128
+        block_size: block wise (128)
+        round_scale: whether round scale to power of 2
+
+    Returns:
+        - y: quantized tensor, float8_e4m3fn
+        - s: quantization scale, float32 [M/128, N/128]
+    """
+    assert x.is_contiguous()
+    assert block_size == 128, "only 128x128 blocks"
+    _lib.require_device_bf16(x, "x")
+    M, N = x.size()
+    assert M % 128 == 0 and N % 128 == 0
+    y = torch.empty((M, N), dtype=fp8_dtype, device=x.device)
+    s = torch.empty(M // block_size, N // block_size, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib.fq_block_quant(_lib.ptr(x), _lib.ptr(y), _lib.ptr(s), M, N, int(bool(round_scale)),
+                                           _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
+    return y, s
+
+
 def triton_blockwise_quant(x, round_scale=False, output_mode=2, *, fp8_dtype=torch.float8_e4m3fn):
     """
     blockwise quantization, used in blockwise recipe in megatron

@@ -30,6 +30,62 @@ def _weight_flag(weight: torch.Tensor) -> int:
     raise TypeError(f"weight must be float32 or bfloat16, got {weight.dtype}")
 
 
+def triton_weighted_silu_forward(x, weight=None, out=None, asm=False):
+    """
+    compute silu(x)*weight, used in bf16/fp16 training with MoE
+    Args:
+        x: input tensor, bf16 [M, 2n] (gate | up)
+        weight: tokenwise weight [M, 1] or [M], fp32 or bf16
+        asm: accepted for compatibility (the reference's alternative exp2 path); ignored
+    Returns:
+        out: output tensor, bf16 [M, n]
+    """
+    assert x.is_contiguous()
+    _lib.require_device_bf16(x, "x")
+    M, N = x.shape
+    assert N % 256 == 0
+    if out is None:
+        out = torch.empty((M, N // 2), device=x.device, dtype=x.dtype)
+    wflag = 0
+    if weight is not None:
+        assert weight.is_contiguous() and weight.numel() == M
+        wflag = _weight_flag(weight)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib.fq_swiglu_fwd(_lib.ptr(x), _lib.ptr(weight), wflag, _lib.ptr(out), M, N // 2,
+                                          _lib.stream_of(x)))
+    return out
+
+
+def triton_weighted_silu_backward(g, x, weight=None):
+    """
+    backward of triton_weighted_silu_forward
+    Args:
+        g: gradient tensor, bf16 [M, n]
+        x: input tensor, bf16 [M, 2n]
+        weight: weight tensor [M, 1] or [M]
+
+    Returns:
+        - dx: gradient of x, bf16 [M, 2n]
+        - dw: gradient of weight (weight's shape and dtype), None without weight
+    """
+    assert g.is_contiguous() and x.is_contiguous()
+    _lib.require_device_bf16(x, "x")
+    _lib.require_device_bf16(g, "g")
+    M, N = x.shape
+    assert N % 256 == 0
+    assert g.shape == (M, N // 2)
+    dw, wflag = None, 0
+    if weight is not None:
+        assert weight.is_contiguous() and weight.numel() == M
+        wflag = _weight_flag(weight)
+        dw = torch.empty(weight.shape, device=x.device, dtype=weight.dtype)
+    dx = torch.empty((M, N), device=x.device, dtype=x.dtype)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib.fq_swiglu_bwd(_lib.ptr(g), _lib.ptr(x), _lib.ptr(weight), wflag, _lib.ptr(dx),
+                                          _lib.ptr(dw), M, N // 2, _lib.stream_of(x)))
+    return dx, dw
+
+
 def triton_silu_and_block_quant_forward(
     x, out=None, scale=None, round_scale=False, output_mode=2, *, fp8_dtype=torch.float8_e4m3fn
 ):

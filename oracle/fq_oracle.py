@@ -22,6 +22,8 @@ reference holds no golden vectors for this path):
   (gradcheck) and against torch.nn.RMSNorm; a dropped 1/n, a wrong power of r
   or a transposed operand fails them.
 * ``swiglu_*`` - closed-form derivatives checked against fp64 autograd.
+* ``block_quant_128`` - per-element loop over the block index formula on a tiny
+  matrix with the same scale/code helpers.
 * ``batch_block_pad_permute_with_indices`` / ``pad_indices`` - element-by-element
   loops over the kernel's published offsets (padded expert starts, padded
   strides, zero padding rows with the floor scale) on a tiny ragged case.
@@ -203,6 +205,22 @@ def silu_and_block_quant_backward(dy, x, round_scale: bool = False, fp8_dtype=E4
     scale [2n/128, M], dx^T codes [2n, M], tscale [ceil(M/128), 2n]."""
     dx, _ = swiglu_grad_fp32(dy, x)
     return blockwise_quant(dx, round_scale, fp8_dtype)
+
+
+def block_quant_128(w, round_scale: bool = False, fp8_dtype=E4M3):
+    """One scale per 128x128 block (linghe/tools/util.py:85-98): amax of the block
+    / fmax, optional power-of-two rounding, true division, RNE cast.  The floor
+    max(scale, 1e-30) is the kernel's (linghe/quant/block.py:24); the reference's
+    torch helper has none and divides an all-zero block by zero.
+    Returns (codes [M,N], scale [M/128, N/128])."""
+    M, N = w.shape
+    wp = w.float().reshape(M // GROUP, GROUP, N // GROUP, GROUP).permute(0, 2, 1, 3)
+    scale = torch.amax(torch.amax(wp.abs(), dim=2), dim=2) / fp8_max(fp8_dtype)
+    scale = torch.maximum(scale, torch.full((1,), SCALE_FLOOR, dtype=torch.float32))
+    if round_scale:
+        scale = _pow2_ceil(scale)
+    q = (wp / scale[:, :, None, None]).to(fp8_dtype)
+    return q.permute(0, 2, 1, 3).reshape(M, N).contiguous(), scale
 
 
 # ----------------------------------------------------------------------------

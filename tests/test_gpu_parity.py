@@ -387,3 +387,60 @@ def test_batch_weighted_silu_bf16_weight_many_experts(gpu):
     announce("batched silu+quant bf16 weight, 300 experts")
     counts = zipf_counts(6000, 300, seed=5, n_empty=7)
     _batched_case(gpu, counts, 512, 1.0, 1.0, seed=34, wdtype=torch.bfloat16)
+
+
+# ------------------------------------------------------------------ bf16 SwiGLU, weight block quant
+@pytest.mark.parametrize("M,N,coef", [(4096, 4096, 1.0), (1000, 1536, 1.0), (33, 256, 10.0), (512, 8192, 0.0)])
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16, None])
+def test_weighted_silu(gpu, M, N, coef, wdtype):
+    """reference tests/test_silu.py:299-329 (x randn, weight randn [M,1], grad randn)."""
+    from linghe_amd.utils.silu import triton_weighted_silu_backward as bwd, triton_weighted_silu_forward as fwd
+
+    announce("weighted silu bf16", M, N, coef, wdtype)
+    g = gen(41)
+    x = randn_bf16(g, M, N, scale=coef)
+    dy = randn_bf16(g, M, N // 2)
+    w = None if wdtype is None else torch.randn(M, 1, generator=g).to(wdtype)
+    y_ref = O.weighted_silu_forward(x, None if w is None else w.float())
+    xd, dyd = _dev(x, gpu), _dev(dy, gpu)
+    wd = None if w is None else _dev(w, gpu)
+    y = fwd(xd, wd)
+    y_asm = fwd(xd, wd, asm=True, out=torch.empty_like(y))
+    torch.cuda.synchronize()
+    assert y.shape == (M, N // 2) and y.dtype == torch.bfloat16
+    check_bf16("wsilu.y", y_ref, y)
+    assert torch.equal(y.cpu().view(torch.int16), y_asm.cpu().view(torch.int16))
+    dx_ref, dw_ref = O.weighted_silu_backward(dy, x, None if w is None else w.float())
+    dx, dw = bwd(dyd, xd, wd)
+    torch.cuda.synchronize()
+    assert dx.shape == (M, N)
+    check_bf16("wsilu.dx", dx_ref, dx)
+    if w is None:
+        assert dw is None
+    else:
+        assert dw.shape == w.shape and dw.dtype == w.dtype
+        tol = 2e-2 if wdtype == torch.bfloat16 else 1e-4
+        torch.testing.assert_close(dw.cpu().float(), dw_ref.float(), rtol=tol,
+                                   atol=tol * max(float(dw_ref.abs().max()), 1e-30))
+
+
+@pytest.mark.parametrize("M,N", [(8192, 4096), (128, 128), (256, 1536)])
+@pytest.mark.parametrize("round_scale", [True, False])
+def test_block_quant(gpu, M, N, round_scale):
+    """reference tests/test_blockwise_quant.py:46-56 (x = randn**3)."""
+    from linghe_amd.quant.block import triton_block_quant
+
+    announce("block_quant 128x128", M, N, round_scale)
+    g = gen(42)
+    x = (torch.randn(M, N, generator=g) ** 3).to(torch.bfloat16)
+    if M >= 256:
+        x[128:256, :128] = 0.0
+    q_ref, s_ref = O.block_quant_128(x, round_scale)
+    q, s = triton_block_quant(_dev(x, gpu), round_scale=round_scale)
+    torch.cuda.synchronize()
+    assert s.shape == (M // 128, N // 128)
+    check_quant_pair("block128", q_ref, s_ref, q, s, **EXACT)
+    q5, s5 = triton_block_quant(_dev(x, gpu), round_scale=round_scale, fp8_dtype=E5M2)
+    torch.cuda.synchronize()
+    r5 = O.block_quant_128(x, round_scale, E5M2)
+    check_quant_pair("block128.e5m2", r5[0], r5[1], q5, s5, **EXACT)

@@ -226,6 +226,27 @@ def test_batched_layouts_elementwise(counts):
     assert float(s2[s0 * nb]) == group_amax_scale(xs.float().numpy()[s0, :128])
 
 
+def test_block_quant_128_elementwise():
+    g = torch.Generator().manual_seed(78)
+    w = (torch.randn(256, 384, generator=g) ** 3).to(torch.bfloat16)
+    w[128:, 128:256] = 0.0  # an all-zero block: floor scale, zero codes
+    q, s = O.block_quant_128(w, round_scale=False)
+    assert s.shape == (2, 3)
+    wf = w.float().numpy()
+    qf = q.float().numpy()
+    for rb in range(2):
+        for cb in range(3):
+            blk = wf[rb * 128:(rb + 1) * 128, cb * 128:(cb + 1) * 128]
+            sc = group_amax_scale(blk.reshape(-1))
+            assert float(s[rb, cb]) == sc
+            for (i, j) in ((0, 0), (5, 127), (127, 64)):
+                want = float(torch.tensor(blk[i, j] / sc).to(torch.float8_e4m3fn).float())
+                assert qf[rb * 128 + i, cb * 128 + j] == want
+    assert float(s[1, 1]) == np.float32(1e-30) and float(q[128:, 128:256].float().abs().max()) == 0.0
+    q2, s2 = O.block_quant_128(w, round_scale=True)
+    assert torch.equal(s2, O._pow2_ceil(s))
+
+
 def test_pad_permute_layouts_elementwise():
     """gather + pad-to-16 + quant against the offsets the reference kernel writes
     (linghe/utils/gather.py:871-940): region start psi = sum of padded counts,
