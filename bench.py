@@ -343,6 +343,40 @@ def build_cases(names, dev):
 
     add("next_block_quant", build=block_quant_case)
 
+    # ---------------------------------------------------------------- next row: RMSNorm + router GEMM + quant
+    def router_case():
+        M, N, K = 8192, 256, 2048
+        g = torch.Generator().manual_seed(1104)
+        x_cpu = (torch.randn(M, K, generator=g) ** 2).to(torch.bfloat16)
+        nw_cpu = torch.randn(K, generator=g).to(torch.bfloat16)
+        rw_cpu = torch.randn(N, K, generator=g).to(torch.bfloat16)
+        nwd, rwd = nw_cpu.to(dev), rw_cpu.to(dev)
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), y=torch.empty((M, K), device=dev, dtype=torch.bfloat16),
+                     r=torch.empty((M,), device=dev, dtype=torch.float32),
+                     lg=torch.empty((M, N), device=dev, dtype=torch.float32),
+                     q=torch.empty((M, K), device=dev, dtype=FP8),
+                     s=torch.empty((K // 128, M), device=dev, dtype=torch.float32))
+            s["ws"] = torch.empty_like(rwd)
+            s["args"] = (_p(s["x"]), _p(nwd), _p(rwd), _p(s["ws"]), _p(s["y"]), _p(s["r"]), _p(s["lg"]), _p(s["q"]), _p(s["s"]),
+                         M, K, N, 1e-6, 0, _lib.FQ_E4M3, stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_rmsnorm_router_quant_fwd(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.rms_gemm_block_quant_forward(x_cpu, nw_cpu, rw_cpu)
+
+        c = Case("next_router", "triton_rms_norm_fp32_gemm_block_quant_forward(output_mode=0)", [M, N, K],
+                 5 * M * K + 4 * M * N + 4 * (K // 128) * M + 4 * M + 2 * N * K + 2 * K, make_set, launch, cpu_fn)
+        c.extra = {"gemm_flops": 2 * M * N * K}
+        return c
+
+    add("next_router", build=router_case)
+
     # ---------------------------------------------------------------- plain copy of known size
     # (calibration of the FETCH_SIZE / WRITE_SIZE counters: reads and writes 256 MiB)
     def copy_case():
@@ -403,7 +437,7 @@ def time_cpu(case, budget_s):
 CFG1_MEASURED_TRAFFIC_BYTES = 102.48e6
 
 ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c", "next_permute",
-       "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant"]
+       "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router"]
 
 
 def main():

@@ -35,6 +35,7 @@ SIGNATURES = {
     "fq_rmsnorm_fwd": [_P, _P, _P, _P, _L, _L, _F, _I, _P],
     "fq_rmsnorm_bwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _P],
     "fq_rmsnorm_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _I, _I, _P, _L, _P],
+    "fq_rmsnorm_router_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _I, _P],
     "fq_swiglu_quant_fwd": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_swiglu_quant_bwd": [_P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_swiglu_quant_fwd": [_P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],

@@ -57,4 +57,9 @@ hipError_t launch_swiglu_rows_bwd(const void* g, const void* x, const void* weig
 hipError_t launch_block_quant(const void* x, void* q, float* s, int64_t M, int N, int round_scale, int kind,
                               hipStream_t stream);
 
+// RMSNorm + router GEMM (N <= 512 logits per row) + 1x128 quant; M a multiple of 32
+hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, void* wpacked, void* y,
+                                       float* rstd, float* logits, void* q, float* s, int64_t M, int K, int N,
+                                       float eps, int round_scale, int kind, hipStream_t stream);
+
 }  // namespace fq

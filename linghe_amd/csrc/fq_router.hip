@@ -1,0 +1,283 @@
+// RMSNorm + router GEMM + 1x128 quant in one pass over x
+// (linghe/utils/norm.py:616-784, output_mode 0; kernel :616-687):
+//   r = rsqrt(mean(x^2) + eps);  y = (x*r)*gamma  (fp32)
+//   y_bf16 = bf16(y);  logits = y @ W^T (fp32);  q, s = 1x128 quant of y
+//
+// The only contraction on this path, so the only place MFMA is used.  The
+// reference multiplies fp32 y by W with tl.dot; here y is split into two bf16
+// terms, y = hi + lo (hi = bf16(y) is the y_bf16 output itself, lo = bf16(y - hi),
+// what is left is below 2^-17 |y|), W is bf16 already, and the two products go
+// through v_mfma_f32_32x32x16_bf16 with fp32 accumulation: bf16 products are
+// exact in fp32, so the result carries the accuracy of an fp32 GEMM at the bf16
+// MFMA rate.
+//
+// One workgroup (4 waves) owns 32 rows and all N <= 512 logits of them and walks K
+// in blocks of 128 (one quantisation group per row):
+//   each thread normalises 2 rows x 8 columns of the block (16 lanes per row, so
+//   every global access is coalesced), quantises them with the row's 1x128 scale
+//   (a DPP reduction over the 16 lanes), stores y_bf16 and the codes, and writes
+//   the hi/lo A operands to LDS in MFMA lane order; after one barrier each wave
+//   multiplies the whole 32x128 block by its N/4 columns of W.
+// Lane l of a wave holds, as MFMA wants it, row l%32 and 8 consecutive k of a
+// 16-wide k step.  Which 16 of the block's 128 columns form step j is free as long
+// as A and B agree: step j takes columns 8j..8j+7 (lanes 0-31) and 64+8j..64+8j+7
+// (lanes 32-63), so that a lane's eight B loads of a block cover one contiguous
+// 128-byte line of its W row; the 32x32 result has column l%32 and rows
+// (v/4)*8 + (l/32)*4 + v%4 in register v.
+#include "fq_device.cuh"
+#include "fq_launch.h"
+
+namespace fq {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kRouterRows = 32;
+
+struct RouterShared {
+  uint4 a[2][2][8][64];  // [buffer][hi, lo][k step][lane slot]: A operands of one 32x128 block
+  float rstd[kRouterRows];
+};
+
+// 1/sqrt(mean(x^2) + eps) of four consecutive rows by one wave (their loads in
+// flight together), the arithmetic of the row kernels: 8-element group sums added
+// in double, so the value does not depend on the split
+__device__ __forceinline__ void router_rows_rstd(const uint16_t* rows, int n, float eps, float (&out)[4]) {
+  const int lane = threadIdx.x & 63;
+  const int chunks = n >> 3;
+  double ss[4] = {0.0, 0.0, 0.0, 0.0};
+  for (int c0 = 0; c0 < chunks; c0 += 256) {
+    uint4 v[4][4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * 64 + lane;
+        v[k][u] = make_uint4(0, 0, 0, 0);
+        if (c < chunks) v[k][u] = *(const uint4*)(rows + (int64_t)k * n + c * 8);
+      }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) ss[k] += (double)sumsq8(v[k][u]);
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) out[k] = 1.0f / sqrtf((float)wave_sum_d(ss[k]) / (float)n + eps);
+}
+
+// W [N, K] -> B operands in the order the main kernel reads them: one 16-byte piece
+// per (k block, wave, column tile, k step, lane), so that every B load of a wave is
+// 1 KB of contiguous memory.  (Read straight from the row-major matrix, each lane of
+// such a load would touch a cache line of its own.)
+__global__ __launch_bounds__(256) void pack_router_weight_kernel(const uint16_t* __restrict__ wr,
+                                                                 uint4* __restrict__ packed, int K, int N) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // piece number
+  const int64_t total = (int64_t)N * K / 8;
+  if (idx >= total) return;
+  const int nt = N / kGroup;
+  const int lane = (int)(idx & 63);
+  int64_t rest = idx >> 6;
+  const int j = (int)(rest & 7);
+  rest >>= 3;
+  const int t = (int)(rest % nt);
+  rest /= nt;
+  const int wave = (int)(rest & 3);
+  const int kb = (int)(rest >> 2);
+  const int n = (wave * nt + t) * 32 + (lane & 31);
+  const int k = kb * kGroup + (lane >> 5) * 64 + j * 8;
+  packed[idx] = *(const uint4*)(wr + (int64_t)n * K + k);
+}
+
+template <int KIND, bool ROUND, int NT>
+__global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma, const uint4* __restrict__ wpacked,
+    uint16_t* __restrict__ y, float* __restrict__ rstd_out, float* __restrict__ logits, uint8_t* __restrict__ q,
+    float* __restrict__ s, int64_t M, int K, int N, float eps) {
+  __shared__ RouterShared sh;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t row0 = (int64_t)blockIdx.x * kRouterRows;
+
+  // ---- statistic of the 32 rows, 8 per wave
+#pragma unroll 1
+  for (int u = 0; u < kRouterRows / 4; u += 4) {
+    const int r = wave * (kRouterRows / 4) + u;
+    float rs[4];
+    router_rows_rstd(x + (row0 + r) * K, K, eps, rs);
+    if (lane < 4) {
+      const float mine = lane == 0 ? rs[0] : lane == 1 ? rs[1] : lane == 2 ? rs[2] : rs[3];
+      sh.rstd[r + lane] = mine;
+      rstd_out[row0 + r + lane] = mine;
+    }
+  }
+  __syncthreads();
+
+  // producer side: thread (rg, cg) holds rows 2 rg, 2 rg + 1 and columns 8 cg .. 8 cg + 7
+  // of the k block, so 16 lanes read, and write, 256 (128 for the codes) contiguous bytes
+  const int cg = threadIdx.x & 15;
+  const int rg = threadIdx.x >> 4;
+  const float r0 = sh.rstd[2 * rg], r1 = sh.rstd[2 * rg + 1];
+  const uint16_t* xrow = x + (row0 + 2 * rg) * K + cg * 8;
+  uint16_t* yrow = y + (row0 + 2 * rg) * K + cg * 8;
+  uint8_t* qrow = q + (row0 + 2 * rg) * K + cg * 8;
+  // consumer side (MFMA lane order)
+  const int arow = lane & 31;
+  const int half = lane >> 5;
+  floatx16_t acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+  const int kblocks = K / kGroup;
+  // operands of a k block: this wave's NT column tiles of W (B operands), the
+  // thread's two rows of x and its piece of gamma.  Only one workgroup of these fits
+  // a CU's share of the rows, so the next block's operands are fetched while the
+  // current one is worked on.
+  auto fetch_w = [&](int kb, uint4 (&b)[NT][8]) {
+    const uint4* wp = wpacked + ((int64_t)(kb * 4 + wave) * NT) * 8 * 64 + lane;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) b[t][j] = wp[(t * 8 + j) * 64];
+  };
+  auto fetch_x = [&](int kb, uint4 (&xr)[2], uint4& gr) {
+    xr[0] = *(const uint4*)(xrow + kb * kGroup);
+    xr[1] = *(const uint4*)(xrow + K + kb * kGroup);
+    gr = *(const uint4*)(gamma + kb * kGroup + cg * 8);
+  };
+  // x comes from HBM (its second read may still find it in a cache), W from L2: x is
+  // fetched kAhead blocks ahead, W one block ahead
+  constexpr int kAhead = 4;
+  uint4 b[NT][8], xq[kAhead][2], gq[kAhead];
+  fetch_w(0, b);
+#pragma unroll
+  for (int d = 0; d < kAhead; ++d)
+    if (d < kblocks) fetch_x(d, xq[d], gq[d]);
+  // column chunk cg of the block is k step (cg & 7), lanes 32*(cg >> 3).. of the A
+  // operand; the row position is XORed with the k step so that the 16-byte LDS
+  // writes of the eight lanes of a row group fall into different banks
+  const int aj = cg & 7;
+  const int ahalf = cg >> 3;
+#pragma unroll 1
+  for (int kb = 0; kb < kblocks; ++kb) {
+    const int buf = kb & 1;
+    uint4 bn[NT][8];
+    uint4 xn[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)}, gn = make_uint4(0, 0, 0, 0);
+    if (kb + 1 < kblocks) fetch_w(kb + 1, bn);
+    if (kb + kAhead < kblocks) fetch_x(kb + kAhead, xn, gn);
+    uint4 xr[2] = {xq[0][0], xq[0][1]};
+    float g[8];
+    unpack8(gq[0], g);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const float r = u ? r1 : r0;
+      float a[8], yv[8];
+      unpack8(xr[u], a);
+      float m = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        yv[i] = (a[i] * r) * g[i];
+        m = fmaxf(m, fabsf(yv[i]));
+      }
+      m = row16_max(m);
+      const float sc = make_scale<KIND, ROUND>(m);
+      const Divisor d = make_divisor(sc);
+      const uint4 hi = pack8_bf16(yv);
+      float back[8], lo[8], qv[8];
+      unpack8(hi, back);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        lo[i] = yv[i] - back[i];
+        qv[i] = div_by_scale<ROUND>(yv[i], d);
+      }
+      const int slot = ahalf * 32 + ((2 * rg + u) ^ aj);
+      sh.a[buf][0][aj][slot] = hi;
+      sh.a[buf][1][aj][slot] = pack8_bf16(lo);
+      *(uint4*)(yrow + (int64_t)u * K + kb * kGroup) = hi;
+      uint2 pk;
+      pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+      pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+      *(uint2*)(qrow + (int64_t)u * K + kb * kGroup) = pk;
+      if (cg == 0) s[(int64_t)kb * M + row0 + 2 * rg + u] = sc;
+    }
+    __syncthreads();
+    // logits += block @ W_block^T
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int slot = half * 32 + (arow ^ j);
+      const bf16x8_t ahi = __builtin_bit_cast(bf16x8_t, sh.a[buf][0][j][slot]);
+      const bf16x8_t alo = __builtin_bit_cast(bf16x8_t, sh.a[buf][1][j][slot]);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, b[t][j]);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi, bw, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo, bw, acc[t], 0, 0, 0);
+      }
+    }
+    if (kb + 1 < kblocks) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) b[t][j] = bn[t][j];
+#pragma unroll
+      for (int d = 0; d + 1 < kAhead; ++d) {
+        xq[d][0] = xq[d + 1][0];
+        xq[d][1] = xq[d + 1][1];
+        gq[d] = gq[d + 1];
+      }
+      xq[kAhead - 1][0] = xn[0];
+      xq[kAhead - 1][1] = xn[1];
+      gq[kAhead - 1] = gn;
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int col = (wave * NT + t) * 32 + arow;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = (v / 4) * 8 + half * 4 + (v % 4);
+      logits[(row0 + row) * N + col] = acc[t][v];
+    }
+  }
+}
+
+hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, void* wpacked, void* y,
+                                       float* rstd, float* logits, void* q, float* s, int64_t M, int K, int N,
+                                       float eps, int round_scale, int kind, hipStream_t stream) {
+  if (M == 0) return hipSuccess;
+  {
+    const int64_t pieces = (int64_t)N * K / 8;
+    hipLaunchKernelGGL(pack_router_weight_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, stream,
+                       (const uint16_t*)wr, (uint4*)wpacked, K, N);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  const dim3 grid((unsigned)(M / kRouterRows)), block(256);
+  const int nt = N / kGroup;
+#define FQ_ROUTER(NTV)                                                                                          \
+  FQ_ROUTER_KIND(NTV)
+#define FQ_ROUTER_KIND(NTV)                                                                                     \
+  if (kind == kE5M2) {                                                                                          \
+    if (round_scale) FQ_ROUTER_GO(kE5M2, true, NTV) else FQ_ROUTER_GO(kE5M2, false, NTV)                        \
+  } else {                                                                                                      \
+    if (round_scale) FQ_ROUTER_GO(kE4M3, true, NTV) else FQ_ROUTER_GO(kE4M3, false, NTV)                        \
+  }
+#define FQ_ROUTER_GO(KINDV, ROUNDV, NTV)                                                                        \
+  { hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, NTV>), grid, block, 0, stream,               \
+                       (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)wpacked, (uint16_t*)y, rstd,     \
+                       logits, (uint8_t*)q, s, M, K, N, eps); }
+  switch (nt) {
+    case 1: FQ_ROUTER(1) break;
+    case 2: FQ_ROUTER(2) break;
+    case 3: FQ_ROUTER(3) break;
+    case 4: FQ_ROUTER(4) break;
+    default: return hipErrorInvalidValue;
+  }
+#undef FQ_ROUTER
+#undef FQ_ROUTER_KIND
+#undef FQ_ROUTER_GO
+  return hipGetLastError();
+}
+
+}  // namespace fq

@@ -109,8 +109,14 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
   const int cg = tid & 15;
   const int rg = tid >> 4;
 
+  // A wave owns 4*RPT consecutive rows.  In a partial tile the waves whose rows all
+  // lie beyond the last stored row have nothing to quantise: their values are
+  // zero, their row-wise outputs do not exist and their bytes of the transposed
+  // tile are never stored, so they only keep the barriers company.
+  const bool live = FULL || wave * (4 * RPT) < o.rows_valid;
+
   // ------------------------------------------------------------- row-wise
-  if constexpr (MODE == 0 || MODE == 2) {
+  if (MODE == 0 || MODE == 2) if (live) {
     // every lane of a 16-lane row gets the amax of its RPT rows; lane cg < RPT then
     // turns ONE of them (row rg*RPT+cg) into {scale, 1/scale}, stores the scale,
     // and hands the pair to the other lanes through LDS.  The rows of a wave are
@@ -156,11 +162,15 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
   if constexpr (MODE == 1 || MODE == 2) {
     float cm[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float m = 0.f;
+    for (int j = 0; j < 8; ++j) cm[j] = 0.f;
+    if (live) {
 #pragma unroll
-      for (int s = 0; s < RPT; ++s) m = fmaxf(m, fabsf(v[s][j]));
-      cm[j] = max_across_rows(m);
+      for (int j = 0; j < 8; ++j) {
+        float m = 0.f;
+#pragma unroll
+        for (int s = 0; s < RPT; ++s) m = fmaxf(m, fabsf(v[s][j]));
+        cm[j] = max_across_rows(m);
+      }
     }
     if (lane < 16) {
       float4* dst = (float4*)&sh.colmax[wave][cg * 8];
@@ -178,6 +188,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       (o.st + o.st_off)[(uint32_t)tid] = sc;
     }
     __syncthreads();
+    if (live) {
     Divisor cd[8];
     {
       const float4* src = (const float4*)&sh.cdiv[cg * 8];
@@ -207,6 +218,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       } else {
         *(uint32_t*)p = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
       }
+    }
     }
     __syncthreads();
     // each transposed row (one column, 128 row-bytes) leaves as 8 x 16 bytes

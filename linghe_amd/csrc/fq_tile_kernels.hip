@@ -109,20 +109,26 @@ __global__ __launch_bounds__(256) void silu_quant_fwd_kernel(const uint16_t* __r
   const int rg = threadIdx.x >> 4;
   float v[RPT][8];
 #pragma unroll
-  for (int s = 0; s < RPT; ++s) {
-    float a[8], b[8];
-    unpack8(r1[s], a);
-    unpack8(r2[s], b);
-    float w = 1.0f;
-    if constexpr (WEIGHTED) {
-      const int i = rg * RPT + s;
-      w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
-    }
+  for (int s = 0; s < RPT; ++s)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float y = (sigmoid_f32(a[j]) * a[j]) * b[j];
-      if constexpr (WEIGHTED) y = y * w;
-      v[s][j] = y;
+    for (int j = 0; j < 8; ++j) v[s][j] = 0.f;
+  if ((threadIdx.x >> 6) * (4 * RPT) < g.rows_valid) {  // waves beyond the last row of a partial tile keep zeros
+#pragma unroll
+    for (int s = 0; s < RPT; ++s) {
+      float a[8], b[8];
+      unpack8(r1[s], a);
+      unpack8(r2[s], b);
+      float w = 1.0f;
+      if constexpr (WEIGHTED) {
+        const int i = rg * RPT + s;
+        w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float y = (sigmoid_f32(a[j]) * a[j]) * b[j];
+        if constexpr (WEIGHTED) y = y * w;
+        v[s][j] = y;
+      }
     }
   }
   quantize_tile<KIND, ROUND, MODE, RPT>(v, make_out(out, g, n, g.cb), sh);
@@ -156,31 +162,37 @@ __global__ __launch_bounds__(512) void silu_quant_bwd_kernel(const uint16_t* __r
   float d1[RPT][8], d2[RPT][8];
   float my_dw = 0.f;
 #pragma unroll
-  for (int s = 0; s < RPT; ++s) {
-    float a[8], b[8], go[8];
-    unpack8(r1[s], a);
-    unpack8(r2[s], b);
-    unpack8(rgd[s], go);
-    float w = 1.0f;
-    const int i = rg * RPT + s;
-    if constexpr (BATCHED) w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
-    float dw = 0.f;
+  for (int s = 0; s < RPT; ++s)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float sg = sigmoid_f32(a[j]);
-      const float sx = sg * a[j];
-      float gw = go[j];
-      if constexpr (BATCHED) {
-        dw += go[j] * (sx * b[j]);
-        gw = go[j] * w;
+    for (int j = 0; j < 8; ++j) d1[s][j] = d2[s][j] = 0.f;
+  if ((threadIdx.x >> 6) * (4 * RPT) < g.rows_valid) {  // waves beyond the last row of a partial tile keep zeros
+#pragma unroll
+    for (int s = 0; s < RPT; ++s) {
+      float a[8], b[8], go[8];
+      unpack8(r1[s], a);
+      unpack8(r2[s], b);
+      unpack8(rgd[s], go);
+      float w = 1.0f;
+      const int i = rg * RPT + s;
+      if constexpr (BATCHED) w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
+      float dw = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float sg = sigmoid_f32(a[j]);
+        const float sx = sg * a[j];
+        float gw = go[j];
+        if constexpr (BATCHED) {
+          dw += go[j] * (sx * b[j]);
+          gw = go[j] * w;
+        }
+        const float h = gw * b[j];
+        d2[s][j] = gw * sx;
+        d1[s][j] = h * sg + ((h * a[j]) * (1.0f - sg)) * sg;
       }
-      const float h = gw * b[j];
-      d2[s][j] = gw * sx;
-      d1[s][j] = h * sg + ((h * a[j]) * (1.0f - sg)) * sg;
-    }
-    if constexpr (BATCHED) {
-      dw = row16_sum(dw);
-      if (cg == s) my_dw = dw;
+      if constexpr (BATCHED) {
+        dw = row16_sum(dw);
+        if (cg == s) my_dw = dw;
+      }
     }
   }
   if constexpr (BATCHED) {

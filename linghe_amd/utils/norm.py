@@ -164,3 +164,71 @@ def triton_rms_norm_and_block_quant_forward(
                 M, n, float(eps), int(bool(round_scale)), output_mode, kind,
                 _lib.ptr(ws), ws_bytes, _lib.stream_of(x)))
     return out, scale, rms, transpose_output, transpose_scale
+
+
+def triton_rms_norm_fp32_gemm_block_quant_forward(
+    x: torch.Tensor,
+    norm_weight: torch.Tensor,
+    route_weight: torch.Tensor,
+    rms: Optional[torch.Tensor] = None,
+    eps: float = 1e-6,
+    output_mode: int = 0,
+    round_scale=False,
+):
+    """
+    y = rms_norm(x)
+    logits = y@w_route
+    x_q, x_s, xt_q, xt_s = quantization(y)
+    Args:
+        x: input tensor, bf16 [M, K]
+        norm weight: weight tensor of rms norm, bf16 [K]
+        route_weight: moe router weight, bf16 [N, K], N in {128, 256, 384, 512}
+        eps: epsilon of rms norm
+        output_mode: 0 or 1
+            0: only output non-transpose quantizatino tensor (and y, rms, logits)
+            1: only output transposed quantizatino tensor (rms must be given)
+
+    Returns:
+        - y: rms normed tensor
+        - rms: 1/rms
+        - logits: router logit
+        - x_q:
+        - x_s:
+        - xt_q:
+        - xt_s:
+    """
+    assert x.is_contiguous() and norm_weight.is_contiguous() and route_weight.is_contiguous()
+    assert output_mode in (0, 1)
+    M, K = x.size()
+    N, K2 = route_weight.size()
+    assert K2 == K
+    assert M % 128 == 0 and K % 128 == 0 and N % 128 == 0
+    _check_hidden(K)
+    _lib.require_device_bf16(x, "x")
+    _lib.require_device_bf16(norm_weight, "norm_weight")
+    device = x.device
+    y = torch.empty(M, K, dtype=x.dtype, device=device)
+    if rms is None:
+        assert output_mode == 0
+        rms = torch.empty(M, dtype=torch.float32, device=device)
+    logits = torch.empty(M, N, dtype=torch.float32, device=device)
+    x_q = torch.empty((M, K), device=device, dtype=torch.float8_e4m3fn)
+    x_s = torch.empty((K // 128, M), device=device, dtype=torch.float32)
+    xt_q = torch.empty((K, M), device=device, dtype=torch.float8_e4m3fn)
+    xt_s = torch.empty((M // 128, K), device=device, dtype=torch.float32)
+    if M == 0:
+        return y, rms, logits, x_q, x_s, xt_q, xt_s
+    with torch.cuda.device(device):
+        if output_mode == 0:
+            _lib.require_device_bf16(route_weight, "route_weight")
+            assert N <= 512, f"{N=} router outputs: at most 512 are supported"
+            scratch = torch.empty_like(route_weight)  # route_weight re-ordered for the matrix cores
+            _lib.check(_lib.lib.fq_rmsnorm_router_quant_fwd(
+                _lib.ptr(x), _lib.ptr(norm_weight), _lib.ptr(route_weight), _lib.ptr(scratch), _lib.ptr(y), _lib.ptr(rms),
+                _lib.ptr(logits), _lib.ptr(x_q), _lib.ptr(x_s), M, K, N, float(eps), int(bool(round_scale)),
+                _lib.FQ_E4M3, _lib.stream_of(x)))
+        else:
+            _lib.check(_lib.lib.fq_rmsnorm_quant_fwd(
+                _lib.ptr(x), _lib.ptr(norm_weight), None, None, _lib.ptr(rms), _lib.ptr(xt_q), _lib.ptr(xt_s),
+                M, K, float(eps), int(bool(round_scale)), 1, _lib.FQ_E4M3, None, 0, _lib.stream_of(x)))
+    return y, rms, logits, x_q, x_s, xt_q, xt_s

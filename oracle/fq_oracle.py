@@ -21,6 +21,8 @@ reference holds no golden vectors for this path):
 * ``rms_norm_*`` - closed forms checked against torch.autograd in fp64
   (gradcheck) and against torch.nn.RMSNorm; a dropped 1/n, a wrong power of r
   or a transposed operand fails them.
+* ``rms_gemm_block_quant_forward`` - composition of the pinned pieces; its GEMM is
+  torch's fp32 matmul, checked against an fp64 product in the pins.
 * ``swiglu_*`` - closed-form derivatives checked against fp64 autograd.
 * ``block_quant_128`` - per-element loop over the block index formula on a tiny
   matrix with the same scale/code helpers.
@@ -160,6 +162,20 @@ def rms_norm_and_block_quant_forward(x, weight, eps: float = 1e-6,
 # ----------------------------------------------------------------------------
 # SwiGLU
 # ----------------------------------------------------------------------------
+def rms_gemm_block_quant_forward(x, norm_weight, route_weight, eps: float = 1e-6,
+                                 round_scale: bool = False, rstd=None):
+    """tests/test_norm.py:87-104: y = fp32 RMSNorm, logits = y @ route_weight^T in
+    fp32, both quantisations of y.  Returns (y in x.dtype, rstd, logits fp32,
+    codes [M,K], scale [K/128, M], transposed codes [K, M], scale [M/128, K])."""
+    y, r = rms_norm_fp32(x, norm_weight, eps)
+    if rstd is not None:  # the statistic the kernel used (see rms_norm_and_block_quant_forward)
+        r = rstd
+        y = (x.float() * r[:, None]) * norm_weight.float()
+    logits = y @ route_weight.float().t()
+    q, s, qt, st = blockwise_quant(y, round_scale)
+    return y.to(x.dtype), r, logits, q, s, qt, st
+
+
 def swiglu_fp32(x: torch.Tensor, row_weight: torch.Tensor | None = None):
     """y = sigmoid(x1) * x1 * x2 [* w_row] in fp32 with x1 | x2 the two halves
     of the last dim (tests/test_silu.py:29-43)."""

@@ -444,3 +444,41 @@ def test_block_quant(gpu, M, N, round_scale):
     torch.cuda.synchronize()
     r5 = O.block_quant_128(x, round_scale, E5M2)
     check_quant_pair("block128.e5m2", r5[0], r5[1], q5, s5, **EXACT)
+
+
+# ------------------------------------------------------------------ RMSNorm + router GEMM + quant
+@pytest.mark.parametrize("M,N,K", [(8192, 256, 2048), (256, 128, 1536), (128, 512, 4096), (384, 384, 7168)])
+@pytest.mark.parametrize("round_scale", [False, True])
+def test_rms_norm_fp32_gemm_block_quant(gpu, M, N, K, round_scale):
+    """reference tests/test_norm.py:251-287 (x = randn**2, weights randn)."""
+    from linghe_amd.utils.norm import triton_rms_norm_fp32_gemm_block_quant_forward as fn
+
+    announce("rmsnorm + router gemm + quant", M, N, K, round_scale)
+    g = gen(24)
+    x = (torch.randn(M, K, generator=g) ** 2).to(torch.bfloat16)
+    nw = torch.randn(K, generator=g).to(torch.bfloat16)
+    rw = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    xd, nwd, rwd = _dev(x, gpu), _dev(nw, gpu), _dev(rw, gpu)
+    y, rms, logits, q, s, qt0, st0 = fn(xd, nwd, rwd, round_scale=round_scale, output_mode=0)
+    torch.cuda.synchronize()
+    assert y.shape == (M, K) and logits.shape == (M, N) and logits.dtype == torch.float32
+    assert s.shape == (K // 128, M) and qt0.shape == (K, M) and st0.shape == (M // 128, K)
+    ref = O.rms_gemm_block_quant_forward(x, nw, rw, round_scale=round_scale)
+    C.assert_scales(ref[1], rms.cpu(), "router.rstd", max_ulp=4, min_within_1ulp=0.9)
+    check_bf16("router.y", ref[0], y)
+    # with the kernel's own statistic everything but the GEMM is bit-exact
+    pin = O.rms_gemm_block_quant_forward(x, nw, rw, round_scale=round_scale, rstd=rms.cpu())
+    assert torch.equal(pin[0].view(torch.int16), y.cpu().view(torch.int16))
+    check_quant_pair("router.row", pin[3], pin[4], q, s, **EXACT)
+    # logits: fp32 GEMM accuracy (the two-term bf16 split leaves < 2^-17 of each |y|;
+    # the reference's own check allows rtol 1e-3, atol 0.1)
+    scale = float((pin[0].float().abs() @ rw.float().abs().t()).max())
+    err = float((logits.cpu() - pin[2]).abs().max())
+    print(f"[parity] router.logits: max abs err {err:.3e}, sum|y||w| max {scale:.3e}", flush=True)
+    assert err <= 2e-5 * scale
+    torch.testing.assert_close(logits.cpu(), ref[2], rtol=1e-3, atol=0.1)
+    # output_mode 1: the transposed copy from the saved statistic
+    _, rms1, _, _, _, qt, st = fn(xd, nwd, rwd, rms=rms, round_scale=round_scale, output_mode=1)
+    torch.cuda.synchronize()
+    assert rms1 is rms
+    check_quant_pair("router.col", pin[5], pin[6], qt, st, **EXACT)

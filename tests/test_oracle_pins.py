@@ -226,6 +226,22 @@ def test_batched_layouts_elementwise(counts):
     assert float(s2[s0 * nb]) == group_amax_scale(xs.float().numpy()[s0, :128])
 
 
+def test_rms_gemm_logits_against_fp64():
+    g = torch.Generator().manual_seed(79)
+    x = (torch.randn(64, 256, generator=g) ** 2).to(torch.bfloat16)
+    w = torch.randn(256, generator=g).to(torch.bfloat16)
+    rw = torch.randn(128, 256, generator=g).to(torch.bfloat16)
+    y16, r, logits, q, s, qt, st = O.rms_gemm_block_quant_forward(x, w, rw)
+    xd = x.double()
+    rd = torch.rsqrt((xd * xd).mean(1) + 1e-6)
+    yd = xd * rd[:, None] * w.double()
+    torch.testing.assert_close(logits.double(), yd @ rw.double().t(), rtol=1e-5, atol=1e-4)
+    torch.testing.assert_close(r.double(), rd, rtol=1e-6, atol=0)
+    assert torch.equal(y16, yd.float().to(torch.bfloat16)) or (y16.float() - yd.float()).abs().max() < 2e-2
+    ref = O.rms_norm_and_block_quant_forward(x, w)
+    assert torch.equal(q.view(torch.uint8), ref[0].view(torch.uint8)) and torch.equal(s, ref[1])
+
+
 def test_block_quant_128_elementwise():
     g = torch.Generator().manual_seed(78)
     w = (torch.randn(256, 384, generator=g) ** 3).to(torch.bfloat16)
