@@ -105,11 +105,11 @@ int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_i
   int rc = check_common(fn, M, N, round_scale, fp8_kind);
   if (rc) return rc;
   if (M == 0) return FQ_OK;  // nothing routed: there is nothing to write (and empty outputs may be NULL)
-  if ((rc = check_mode_ptrs(fn, 2, q, s, qt, st))) return rc;
   FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0 && src_rows >= 0, FQ_ERR_SHAPE, "%s: negative count", fn);
   FQ_REQUIRE(src_rows <= ((int64_t)1 << 31) - 1, FQ_ERR_SHAPE, "%s: too many source rows for int32 indices", fn);
   FQ_REQUIRE(M % 16 == 0, FQ_ERR_SHAPE, "%s: M (%lld) must be the sum of the counts each rounded up to 16", fn,
              (long long)M);
+  if ((rc = check_mode_ptrs(fn, 2, q, s, qt, st))) return rc;
   FQ_REQUIRE((probs == nullptr) == (prob_out == nullptr), FQ_ERR_ARG, "%s: probs and prob_out go together", fn);
   if (M == 0 || total_blocks == 0 || src_rows == 0) return FQ_OK;
   FQ_REQUIRE(x && aligned16(x) && counts && indices && aligned16(indices), FQ_ERR_ARG,

@@ -21,9 +21,9 @@ def triton_block_quant(x, block_size=128, round_scale=False, *, fp8_dtype=torch.
     """
     assert x.is_contiguous()
     assert block_size == 128, "only 128x128 blocks"
-    _lib.require_device_bf16(x, "x")
     M, N = x.size()
     assert M % 128 == 0 and N % 128 == 0
+    _lib.require_device_bf16(x, "x")
     y = torch.empty((M, N), dtype=fp8_dtype, device=x.device)
     s = torch.empty(M // block_size, N // block_size, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):

@@ -63,8 +63,29 @@ def test_c_side_validation_without_gpu():
     # hidden size too large for the row kernels
     rc = L.fq_rmsnorm_fwd(None, None, None, None, 4, 16384, 1e-6, 0, None)
     assert rc == -2
+    # 128x128 block quant needs whole blocks of rows
+    rc = L.fq_block_quant(None, None, None, 100, 256, 0, 0, None)
+    assert rc == -2 and b"128" in L.fq_last_error()
+    # router GEMM: at most 512 outputs, rows in groups of 32
+    rc = L.fq_rmsnorm_router_quant_fwd(None, None, None, None, None, None, None, None, None, 128, 2048, 640, 1e-6, 0, 0,
+                                       None)
+    assert rc == -2 and b"router" in L.fq_last_error()
+    rc = L.fq_rmsnorm_router_quant_fwd(None, None, None, None, None, None, None, None, None, 100, 2048, 256, 1e-6, 0, 0,
+                                       None)
+    assert rc == -2
+    # gather + pad: the output row count is a sum of multiples of 16; probs and prob_out go together
+    rc = L.fq_batched_pad_permute_quant(None, None, 0, 4, 1, None, None, 0, None, None, None, None, None, 64, 100, 256,
+                                        0, 0, None)
+    assert rc == -2 and b"16" in L.fq_last_error()
+    # more rows / wider than the 32-bit lane offsets of a tile allow
+    rc = L.fq_blockwise_quant(None, None, None, None, None, (1 << 24) + 16, 128, 0, 2, 0, None)
+    assert rc == -2
+    # bf16 SwiGLU: weight and dw go together
+    rc = L.fq_swiglu_bwd(None, None, None, 0, None, ctypes.c_void_p(16), 16, 128, None)
+    assert rc == -1
     # empty problem is a no-op
     assert L.fq_group_quant(None, None, None, 0, 128, 0, 0, None) == 0
+    assert L.fq_swiglu_fwd(None, None, 0, None, 0, 128, None) == 0
     with pytest.raises(RuntimeError):
         _lib.check(-2)
 
@@ -91,6 +112,16 @@ REFERENCE_SIGNATURES = {
                                   ["xs", "token_count_per_expert", "splits", "round_scale"]),
     "linghe/quant/group.py:40": ("linghe_amd.quant.group", "triton_group_quant",
                                  ["x", "dtype", "group_size", "round_scale"]),
+    "linghe/quant/block.py:32": ("linghe_amd.quant.block", "triton_block_quant",
+                                 ["x", "block_size", "round_scale"]),
+    "linghe/utils/silu.py:98": ("linghe_amd.utils.silu", "triton_weighted_silu_forward",
+                                ["x", "weight", "out", "asm"]),
+    "linghe/utils/silu.py:177": ("linghe_amd.utils.silu", "triton_weighted_silu_backward",
+                                 ["g", "x", "weight"]),
+    "linghe/utils/gather.py:960": ("linghe_amd.utils.gather", "triton_batch_block_pad_permute_with_indices",
+                                   ["xs", "token_count_per_expert", "indices", "splits", "probs", "round_scale"]),
+    "linghe/utils/norm.py:690": ("linghe_amd.utils.norm", "triton_rms_norm_fp32_gemm_block_quant_forward",
+                                 ["x", "norm_weight", "route_weight", "rms", "eps", "output_mode", "round_scale"]),
 }
 
 
@@ -123,6 +154,9 @@ def test_host_asserts_fire_on_cpu_tensors():
         triton_blockwise_quant(torch.zeros(17, 256, dtype=torch.bfloat16))  # M % 16
     with pytest.raises(AssertionError):
         triton_blockwise_quant(x.t())  # not contiguous
+    with pytest.raises(AssertionError):
+        from linghe_amd.quant.block import triton_block_quant
+        triton_block_quant(torch.zeros(100, 256, dtype=torch.bfloat16))  # M % 128
     with pytest.raises(AssertionError, match="splits"):
         triton_batch_weighted_silu_and_block_quant_forward(x, torch.zeros(32, 1), torch.zeros(2, dtype=torch.int32))
     with pytest.raises(AssertionError):
