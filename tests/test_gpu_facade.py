@@ -205,3 +205,61 @@ def test_block_batch_weighted_silu(gpu, is_recomputing):
                      gq.kw["columnwise_scale_inv"].view(-1), **FUSED_BWD)
     assert wd.grad.shape == (bs, 1) and wd.grad.dtype == torch.float32
     torch.testing.assert_close(wd.grad.cpu(), rb[2], rtol=1e-4, atol=1e-4 * float(rb[2].abs().max()))
+
+
+def test_entry_points_under_graph_capture(gpu):
+    """The library only enqueues work on the given stream, so its calls can be
+    captured into a graph: every replay (with eager work and synchronisations in
+    between) must reproduce the eager results bit for bit.  With the single-pass
+    switch on, a capturing stream still gets the two-pass kernels."""
+    import linghe_amd.utils.norm as norm_mod
+    from linghe_amd.quant.block import triton_blockwise_quant
+    from linghe_amd.utils.norm import triton_rms_norm_and_block_quant_forward, triton_rms_norm_backward
+    from linghe_amd.utils.silu import (triton_batch_weighted_silu_and_block_quant_forward,
+                                       triton_silu_and_block_quant_backward)
+
+    announce("graph capture and replay")
+    g = gen(55)
+    M, N = 512, 1024
+    x = randn_bf16(g, M, N).to(gpu)
+    x2 = randn_bf16(g, M, N).to(gpu)
+    w = gamma_bf16(g, N).to(gpu)
+    dy = randn_bf16(g, M, N // 2).to(gpu)
+    counts = [100, 0, 156, 256]
+    cnt = torch.tensor(counts, dtype=torch.int32, device=gpu)
+    rw = torch.rand(M, 1, generator=g).to(gpu)
+
+    def run(inp):
+        a = triton_rms_norm_and_block_quant_forward(inp, w)
+        b = triton_silu_and_block_quant_backward(dy, inp)
+        c = triton_batch_weighted_silu_and_block_quant_forward(inp, rw, cnt, counts)
+        d = triton_rms_norm_backward(inp, inp, w)
+        e = triton_blockwise_quant(inp)
+        return [t for grp in (a, b, c, d, e) for t in grp]
+
+    def bits(ts):
+        return [t.detach().clone().view(torch.uint8) if t.dtype != torch.float32 else t.detach().clone() for t in ts]
+
+    eager1, eager2 = bits(run(x)), bits(run(x2))
+    torch.cuda.synchronize()
+    static_in = x.clone()
+    norm_mod.SINGLE_PASS = True
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run(static_in)  # warm-up on the capture stream
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = run(static_in)
+    finally:
+        norm_mod.SINGLE_PASS = False
+    for rep, (src, want) in enumerate(((x, eager1), (x2, eager2), (x, eager1), (x2, eager2))):
+        static_in.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = bits(outs)
+        for k, (a, b) in enumerate(zip(want, got)):
+            assert torch.equal(a, b), (rep, k)
+        _ = (src.float() * 2).sum().item()  # eager work between the replays
