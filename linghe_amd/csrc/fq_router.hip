@@ -66,7 +66,7 @@ __device__ __forceinline__ void router_rows_rstd(const uint16_t* rows, int n, fl
 }
 
 // W [N, K] -> B operands in the order the main kernel reads them: one 16-byte piece
-// per (k block, wave, column tile, k step, lane), so that every B load of a wave is
+// per (k block, 32-column tile, k step, lane), so that every B load of a wave is
 // 1 KB of contiguous memory.  (Read straight from the row-major matrix, each lane of
 // such a load would touch a cache line of its own.)
 __global__ __launch_bounds__(256) void pack_router_weight_kernel(const uint16_t* __restrict__ wr,
@@ -74,22 +74,22 @@ __global__ __launch_bounds__(256) void pack_router_weight_kernel(const uint16_t*
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // piece number
   const int64_t total = (int64_t)N * K / 8;
   if (idx >= total) return;
-  const int nt = N / kGroup;
+  const int tiles = N / 32;
   const int lane = (int)(idx & 63);
   int64_t rest = idx >> 6;
   const int j = (int)(rest & 7);
   rest >>= 3;
-  const int t = (int)(rest % nt);
-  rest /= nt;
-  const int wave = (int)(rest & 3);
-  const int kb = (int)(rest >> 2);
-  const int n = (wave * nt + t) * 32 + (lane & 31);
+  const int tile = (int)(rest % tiles);
+  const int kb = (int)(rest / tiles);
+  const int n = tile * 32 + (lane & 31);
   const int k = kb * kGroup + (lane >> 5) * 64 + j * 8;
   packed[idx] = *(const uint4*)(wr + (int64_t)n * K + k);
 }
 
-template <int KIND, bool ROUND, int NT>
-__global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
+// WAVES waves per workgroup, TPW column tiles (of 32 logits) per wave: N = 32 * WAVES * TPW.
+// With 8 waves a thread owns one row x 8 columns of a k block, with 4 waves two rows.
+template <int KIND, bool ROUND, int TPW, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma, const uint4* __restrict__ wpacked,
     uint16_t* __restrict__ y, float* __restrict__ rstd_out, float* __restrict__ logits, uint8_t* __restrict__ q,
     float* __restrict__ s, int64_t M, int K, int N, float eps) {
@@ -98,10 +98,12 @@ __global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
   const int wave = threadIdx.x >> 6;
   const int64_t row0 = (int64_t)blockIdx.x * kRouterRows;
 
-  // ---- statistic of the 32 rows, 8 per wave
+  constexpr int NT = TPW;
+  constexpr int RPT = 8 / WAVES;  // rows per thread: 2 with 4 waves, 1 with 8
+  // ---- statistic of the 32 rows, four at a time per wave
 #pragma unroll 1
-  for (int u = 0; u < kRouterRows / 4; u += 4) {
-    const int r = wave * (kRouterRows / 4) + u;
+  for (int u = 0; u < kRouterRows / WAVES; u += 4) {
+    const int r = wave * (kRouterRows / WAVES) + u;
     float rs[4];
     router_rows_rstd(x + (row0 + r) * K, K, eps, rs);
     if (lane < 4) {
@@ -112,14 +114,14 @@ __global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
   }
   __syncthreads();
 
-  // producer side: thread (rg, cg) holds rows 2 rg, 2 rg + 1 and columns 8 cg .. 8 cg + 7
-  // of the k block, so 16 lanes read, and write, 256 (128 for the codes) contiguous bytes
+  // producer side: thread (rg, cg) holds rows RPT rg .. and columns 8 cg .. 8 cg + 7 of
+  // the k block, so 16 lanes read, and write, 256 (128 for the codes) contiguous bytes
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
-  const float r0 = sh.rstd[2 * rg], r1 = sh.rstd[2 * rg + 1];
-  const uint16_t* xrow = x + (row0 + 2 * rg) * K + cg * 8;
-  uint16_t* yrow = y + (row0 + 2 * rg) * K + cg * 8;
-  uint8_t* qrow = q + (row0 + 2 * rg) * K + cg * 8;
+  const float r0 = sh.rstd[RPT * rg], r1 = sh.rstd[RPT * rg + RPT - 1];
+  const uint16_t* xrow = x + (row0 + RPT * rg) * K + cg * 8;
+  uint16_t* yrow = y + (row0 + RPT * rg) * K + cg * 8;
+  uint8_t* qrow = q + (row0 + RPT * rg) * K + cg * 8;
   // consumer side (MFMA lane order)
   const int arow = lane & 31;
   const int half = lane >> 5;
@@ -135,42 +137,31 @@ __global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
   // a CU's share of the rows, so the next block's operands are fetched while the
   // current one is worked on.
   auto fetch_w = [&](int kb, uint4 (&b)[NT][8]) {
-    const uint4* wp = wpacked + ((int64_t)(kb * 4 + wave) * NT) * 8 * 64 + lane;
+    const uint4* wp = wpacked + ((int64_t)(kb * WAVES + wave) * NT) * 8 * 64 + lane;
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int j = 0; j < 8; ++j) b[t][j] = wp[(t * 8 + j) * 64];
   };
-  auto fetch_x = [&](int kb, uint4 (&xr)[2], uint4& gr) {
-    xr[0] = *(const uint4*)(xrow + kb * kGroup);
-    xr[1] = *(const uint4*)(xrow + K + kb * kGroup);
+  auto fetch_x = [&](int kb, uint4 (&xr)[RPT], uint4& gr) {
+#pragma unroll
+    for (int u = 0; u < RPT; ++u) xr[u] = *(const uint4*)(xrow + (int64_t)u * K + kb * kGroup);
     gr = *(const uint4*)(gamma + kb * kGroup + cg * 8);
   };
-  // x comes from HBM (its second read may still find it in a cache), W from L2: x is
-  // fetched kAhead blocks ahead, W one block ahead
-  constexpr int kAhead = 4;
-  uint4 b[NT][8], xq[kAhead][2], gq[kAhead];
-  fetch_w(0, b);
-#pragma unroll
-  for (int d = 0; d < kAhead; ++d)
-    if (d < kblocks) fetch_x(d, xq[d], gq[d]);
   // column chunk cg of the block is k step (cg & 7), lanes 32*(cg >> 3).. of the A
   // operand; the row position is XORed with the k step so that the 16-byte LDS
   // writes of the eight lanes of a row group fall into different banks
   const int aj = cg & 7;
   const int ahalf = cg >> 3;
-#pragma unroll 1
-  for (int kb = 0; kb < kblocks; ++kb) {
+
+  // one k block: normalise / quantise / store the thread's piece, publish the A
+  // operands, then multiply the whole block by this wave's columns of W
+  auto step = [&](int kb, const uint4 (&xr)[RPT], const uint4& gr, const uint4 (&b)[NT][8]) {
     const int buf = kb & 1;
-    uint4 bn[NT][8];
-    uint4 xn[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)}, gn = make_uint4(0, 0, 0, 0);
-    if (kb + 1 < kblocks) fetch_w(kb + 1, bn);
-    if (kb + kAhead < kblocks) fetch_x(kb + kAhead, xn, gn);
-    uint4 xr[2] = {xq[0][0], xq[0][1]};
     float g[8];
-    unpack8(gq[0], g);
+    unpack8(gr, g);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < RPT; ++u) {
       const float r = u ? r1 : r0;
       float a[8], yv[8];
       unpack8(xr[u], a);
@@ -191,7 +182,7 @@ __global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
         lo[i] = yv[i] - back[i];
         qv[i] = div_by_scale<ROUND>(yv[i], d);
       }
-      const int slot = ahalf * 32 + ((2 * rg + u) ^ aj);
+      const int slot = ahalf * 32 + ((RPT * rg + u) ^ aj);
       sh.a[buf][0][aj][slot] = hi;
       sh.a[buf][1][aj][slot] = pack8_bf16(lo);
       *(uint4*)(yrow + (int64_t)u * K + kb * kGroup) = hi;
@@ -199,10 +190,9 @@ __global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
       pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
       pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
       *(uint2*)(qrow + (int64_t)u * K + kb * kGroup) = pk;
-      if (cg == 0) s[(int64_t)kb * M + row0 + 2 * rg + u] = sc;
+      if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
     }
     __syncthreads();
-    // logits += block @ W_block^T
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int slot = half * 32 + (arow ^ j);
@@ -215,20 +205,28 @@ __global__ __launch_bounds__(256) void rmsnorm_router_quant_kernel(
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo, bw, acc[t], 0, 0, 0);
       }
     }
-    if (kb + 1 < kblocks) {
+  };
+
+  // x comes from HBM (its second read may still find it in a cache), W from L2: x is
+  // fetched kAhead blocks ahead, W one block ahead.  The loop is unrolled over the
+  // ring of kAhead operand sets so that a set is refilled in place right after it
+  // was used: no register is copied while its load is still in flight.
+  constexpr int kAhead = 4;
+  uint4 b[2][NT][8], xq[kAhead][RPT], gq[kAhead];
+  fetch_w(0, b[0]);
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+  for (int d = 0; d < kAhead; ++d)
+    if (d < kblocks) fetch_x(d, xq[d], gq[d]);
+#pragma unroll 1
+  for (int kb0 = 0; kb0 < kblocks; kb0 += kAhead) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) b[t][j] = bn[t][j];
-#pragma unroll
-      for (int d = 0; d + 1 < kAhead; ++d) {
-        xq[d][0] = xq[d + 1][0];
-        xq[d][1] = xq[d + 1][1];
-        gq[d] = gq[d + 1];
+    for (int d = 0; d < kAhead; ++d) {
+      const int kb = kb0 + d;
+      if (kb < kblocks) {
+        if (kb + 1 < kblocks) fetch_w(kb + 1, b[(d + 1) & 1]);
+        step(kb, xq[d], gq[d], b[d & 1]);
+        if (kb + kAhead < kblocks) fetch_x(kb + kAhead, xq[d], gq[d]);
       }
-      xq[kAhead - 1][0] = xn[0];
-      xq[kAhead - 1][1] = xn[1];
-      gq[kAhead - 1] = gn;
     }
   }
 #pragma unroll
@@ -253,28 +251,26 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
-  const dim3 grid((unsigned)(M / kRouterRows)), block(256);
-  const int nt = N / kGroup;
-#define FQ_ROUTER(NTV)                                                                                          \
-  FQ_ROUTER_KIND(NTV)
-#define FQ_ROUTER_KIND(NTV)                                                                                     \
+  const dim3 grid((unsigned)(M / kRouterRows));
+  const int tiles = N / 32;
+  // 8 waves when the column tiles split evenly over them (N = 256, 512), else 4
+#define FQ_ROUTER_GO(KINDV, ROUNDV, TPWV, WAVESV)                                                               \
+  hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, TPWV, WAVESV>), grid, dim3(64 * WAVESV), 0,    \
+                     stream, (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)wpacked, (uint16_t*)y,   \
+                     rstd, logits, (uint8_t*)q, s, M, K, N, eps)
+#define FQ_ROUTER_KIND(TPWV, WAVESV)                                                                            \
   if (kind == kE5M2) {                                                                                          \
-    if (round_scale) FQ_ROUTER_GO(kE5M2, true, NTV) else FQ_ROUTER_GO(kE5M2, false, NTV)                        \
+    if (round_scale) FQ_ROUTER_GO(kE5M2, true, TPWV, WAVESV); else FQ_ROUTER_GO(kE5M2, false, TPWV, WAVESV);    \
   } else {                                                                                                      \
-    if (round_scale) FQ_ROUTER_GO(kE4M3, true, NTV) else FQ_ROUTER_GO(kE4M3, false, NTV)                        \
+    if (round_scale) FQ_ROUTER_GO(kE4M3, true, TPWV, WAVESV); else FQ_ROUTER_GO(kE4M3, false, TPWV, WAVESV);    \
   }
-#define FQ_ROUTER_GO(KINDV, ROUNDV, NTV)                                                                        \
-  { hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, NTV>), grid, block, 0, stream,               \
-                       (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)wpacked, (uint16_t*)y, rstd,     \
-                       logits, (uint8_t*)q, s, M, K, N, eps); }
-  switch (nt) {
-    case 1: FQ_ROUTER(1) break;
-    case 2: FQ_ROUTER(2) break;
-    case 3: FQ_ROUTER(3) break;
-    case 4: FQ_ROUTER(4) break;
+  switch (tiles) {
+    case 4: FQ_ROUTER_KIND(1, 4) break;
+    case 8: FQ_ROUTER_KIND(1, 8) break;
+    case 12: FQ_ROUTER_KIND(3, 4) break;
+    case 16: FQ_ROUTER_KIND(2, 8) break;
     default: return hipErrorInvalidValue;
   }
-#undef FQ_ROUTER
 #undef FQ_ROUTER_KIND
 #undef FQ_ROUTER_GO
   return hipGetLastError();
