@@ -413,14 +413,36 @@ def time_loop(case, sets, steps, warmup):
     return start.elapsed_time(end) * 1000.0 / steps
 
 
+def time_single_calls(case, sets, calls, warmup):
+    """(median, trimmed mean) in us of event pairs around single calls, the
+    protocol of the reference's own harness (linghe/tools/benchmark.py:32-70:
+    one event pair per call, sorted, max(1, n/100) dropped at either end).  The
+    events' own cost is inside every sample, so these read a few us above the
+    back-to-back figure."""
+    k = len(sets)
+    for i in range(warmup):
+        case.launch(sets[i % k])
+    torch.cuda.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(calls)]
+    for i, (a, b) in enumerate(pairs):
+        a.record()
+        case.launch(sets[i % k])
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) * 1000.0 for a, b in pairs)
+    clip = max(1, calls // 100)
+    kept = t[clip:-clip] if 2 * clip < calls else t
+    return t[len(t) // 2], sum(kept) / len(kept)
+
+
 def time_cpu(case, budget_s):
-    """oracle on the host cores: 1 warm-up, then min over up to 3 runs within the budget."""
+    """oracle on the host cores: 1 warm-up, then min over up to 20 runs within the budget."""
     t0 = time.perf_counter()
     case.cpu_fn()
     first = time.perf_counter() - t0
     runs = [first]
     spent = first
-    while len(runs) < 4 and spent + runs[-1] < budget_s:
+    while len(runs) < 21 and spent + runs[-1] < budget_s:
         t0 = time.perf_counter()
         case.cpu_fn()
         runs.append(time.perf_counter() - t0)
@@ -474,10 +496,12 @@ def main():
             case.sets = case.sets[:1]
         cold = time_loop(case, case.sets, args.steps, args.warmup)
         hot = cold if args.hot_only else time_loop(case, case.sets[:1], args.steps, args.warmup)
+        med, trimmed = time_single_calls(case, case.sets, max(10, min(args.steps, 200)), min(args.warmup, 10))
         gbs = case.algo_bytes / cold / 1e3
         r = dict(entry=case.entry, shape=case.shape, algorithmic_bytes=case.algo_bytes,
                  us_per_call=round(cold, 3), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
                  us_per_call_hot=round(hot, 3), gb_per_s_hot=round(case.algo_bytes / hot / 1e3, 1),
+                 us_single_call_median=round(med, 3), us_single_call_trimmed_mean=round(trimmed, 3),
                  buffer_sets=len(case.sets))
         if hasattr(case, "extra"):
             r.update(case.extra)

@@ -219,16 +219,22 @@ __device__ __forceinline__ double wave_sum_d(double v) {
 }
 
 // sigmoid(x) = 1 / (1 + exp(-x)):
-//   exp(-x) = exp2(x * -log2(e)) with v_exp_f32 (1 ulp); the fp32 product costs up
-//   to |x|*4e-8 of relative error in exp(-x), which only matters where exp(-x) is
-//   large, i.e. where sigmoid (and silu) is small;
-//   the reciprocal is v_rcp_f32 plus one Newton step (correctly rounded but for
+//   exp(-x) = exp2(-x*log2(e)) with v_exp_f32 (1 ulp). A single fp32 product
+//   x * -log2(e) would round the exponent and cost up to |x|*4e-8 of relative error
+//   (11 ulp of the sigmoid at x = -8), so -log2(e) is split into a 16-bit head,
+//   whose product with a bf16-valued x (8 significant bits) is exact, and a tail
+//   applied to first order: exp2(hi + lo) = exp2(hi) * (1 + lo*ln2), |lo*ln2| < 1e-3.
+//   For an x with more than 8 significant bits the head product rounds and the old
+//   bound applies; every caller passes widened bf16 data.
+//   The reciprocal is v_rcp_f32 plus one Newton step (correctly rounded but for
 //   ~1e-6 of the inputs).
 // The exponent is clamped so that 1 + exp(-x) stays finite: for x < -87 the result
 // is 2^-126 instead of 0, far below anything a code or a scale can see.
 __device__ __forceinline__ float sigmoid_f32(float x) {
-  const float t = fminf(x * -1.4426950408889634f, 126.0f);
-  const float d = 1.0f + __builtin_amdgcn_exp2f(t);
+  constexpr float kHead = -1.44268798828125f;         // -log2(e) to 16 significant bits
+  constexpr float kTailLn2 = -4.888495368504664e-06f; // (-log2(e) - kHead) * ln(2)
+  const float e0 = __builtin_amdgcn_exp2f(fminf(x * kHead, 126.0f));
+  const float d = 1.0f + __builtin_fmaf(e0, x * kTailLn2, e0);
   const float r0 = __builtin_amdgcn_rcpf(d);
   const float err = __builtin_fmaf(-d, r0, 1.0f);
   return __builtin_fmaf(err, r0, r0);

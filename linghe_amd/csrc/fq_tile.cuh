@@ -116,7 +116,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
   const bool live = FULL || wave * (4 * RPT) < o.rows_valid;
 
   // ------------------------------------------------------------- row-wise
-  if (MODE == 0 || MODE == 2) if (live) {
+  if ((MODE == 0 || MODE == 2) && live) {
     // every lane of a 16-lane row gets the amax of its RPT rows; lane cg < RPT then
     // turns ONE of them (row rg*RPT+cg) into {scale, 1/scale}, stores the scale,
     // and hands the pair to the other lanes through LDS.  The rows of a wave are
