@@ -1,5 +1,6 @@
 // Device-side building blocks for the fused blockwise-FP8 quantisation kernels
-// (gfx950 / CDNA4, wave64).  No MFMA: every kernel on this path is HBM-bound.
+// (gfx950 / CDNA4, wave64).  No MFMA here: the kernels built on this header are
+// HBM-bound; the one contraction of the path has its own file (fq_router.hip).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -208,11 +209,16 @@ __device__ __forceinline__ double dpp_mov_d(double v) {
   const uint32_t hi = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)(u >> 32), CTRL, 0xf, 0xf, true);
   return __builtin_bit_cast(double, (uint64_t)lo | ((uint64_t)hi << 32));
 }
-__device__ __forceinline__ double wave_sum_d(double v) {
+// every lane of the 16-lane row ends with the same sum
+__device__ __forceinline__ double row16_sum_d(double v) {
   v += dpp_mov_d<kDppQuadXor1>(v);
   v += dpp_mov_d<kDppQuadXor2>(v);
   v += dpp_mov_d<kDppRowHalfMirror>(v);
   v += dpp_mov_d<kDppRowMirror>(v);
+  return v;
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+  v = row16_sum_d(v);
   v += __shfl_xor(v, 16, 64);
   v += __shfl_xor(v, 32, 64);
   return v;

@@ -11,7 +11,11 @@
 // exact in fp32, so the result carries the accuracy of an fp32 GEMM at the bf16
 // MFMA rate.
 //
-// One workgroup (4 waves) owns 32 rows and all N <= 512 logits of them and walks K
+// Two kernels share this scheme: the one below streams the rows twice (statistic,
+// then the blocks) and takes any K; rmsnorm_router_quant_resident_kernel further
+// down keeps the rows in registers when they fit.
+//
+// One workgroup (4 or 8 waves) owns 32 rows and all N <= 512 logits of them and walks K
 // in blocks of 128 (one quantisation group per row):
 //   each thread normalises 2 rows x 8 columns of the block (16 lanes per row, so
 //   every global access is coalesced), quantises them with the row's 1x128 scale
@@ -240,6 +244,183 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
   }
 }
 
+
+// The same operation for K <= 128 * KB with the workgroup's rows of x held in
+// registers, so that x is read from memory once and the GEMM does not wait for the
+// statistic.  rstd is a per-row factor of y, hence of the logits:
+//   logits[r, :] = rstd[r] * sum_k (x[r,k] * gamma[k]) * W[:, k]
+// and z = x * gamma is EXACT in fp32 (two 8-bit significands), as is its split
+// z = hi + lo into two bf16 values, so the contraction carries only the rounding of
+// the fp32 accumulation and one final multiplication by rstd.
+//   sweep 1, per k block as x arrives: z -> hi/lo A operands in LDS -> MFMA; the sum
+//     of squares accumulates beside it (8-element group sums added in double, the
+//     arithmetic of the row kernels); the next block's W loads are issued between
+//     the MFMAs so that the memory pipeline and the matrix cores work together;
+//   sweep 2, from registers: logits *= rstd; y = (x*rstd)*gamma -> bf16, codes and
+//     scales, streamed out.
+template <int KIND, bool ROUND, int TPW, int WAVES, int KB, int WDEPTH>
+__global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma, const uint4* __restrict__ wpacked,
+    uint16_t* __restrict__ y, float* __restrict__ rstd_out, float* __restrict__ logits, uint8_t* __restrict__ q,
+    float* __restrict__ s, int64_t M, int K, int N, float eps) {
+  __shared__ RouterShared sh;
+  __shared__ uint4 sgamma[KB * 16];  // gamma, 8 columns per piece
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t row0 = (int64_t)blockIdx.x * kRouterRows;
+  constexpr int NT = TPW;
+  constexpr int RPT = 8 / WAVES;
+  constexpr int kAhead = 6;  // k blocks of x in flight ahead of the one worked on
+  constexpr int kEarly = 0;  // W pieces requested ahead of the MFMA loop rather than inside it
+  constexpr int kWAhead = WDEPTH - 1;  // k blocks of W in flight ahead of the one worked on
+  const int cg = threadIdx.x & 15;
+  const int rg = threadIdx.x >> 4;
+  const uint16_t* xrow = x + (row0 + RPT * rg) * K + cg * 8;
+  const int aj = cg & 7;
+  const int ahalf = cg >> 3;
+  const int arow = lane & 31;
+  const int half = lane >> 5;
+  const int kblocks = K / kGroup;
+
+  floatx16_t acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+  uint4 xr[KB][RPT], b[WDEPTH][NT][8];
+  double ss[RPT];
+#pragma unroll
+  for (int u = 0; u < RPT; ++u) ss[u] = 0.0;
+  const uint4* wlane = wpacked + (int64_t)wave * NT * 8 * 64 + lane;
+  auto w_piece = [&](int kb, int t, int j) { return wlane[((int64_t)kb * WAVES * NT + t) * 8 * 64 + j * 64]; };
+  auto fetch_x = [&](int kb, uint4 (&xk)[RPT]) {
+#pragma unroll
+    for (int u = 0; u < RPT; ++u) xk[u] = *(const uint4*)(xrow + (int64_t)u * K + kb * kGroup);
+  };
+#pragma unroll
+  for (int d = 0; d < kWAhead; ++d)
+    if (d < kblocks) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) b[d][t][j] = w_piece(d, t, j);
+    }
+#pragma unroll
+  for (int d = 0; d < kAhead; ++d)
+    if (d < KB && d < kblocks) fetch_x(d, xr[d]);
+  for (int p = threadIdx.x; p < kblocks * 16; p += 64 * WAVES) sgamma[p] = *(const uint4*)(gamma + p * 8);
+  __syncthreads();
+
+  // ---- sweep 1
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    if (kb < kblocks) {
+      const int buf = kb & 1;
+      const bool more = kb + kWAhead < kblocks;
+      const int kNext = (kb + kWAhead) % WDEPTH;
+      // the next block's W: the first kEarly pieces are requested before this block's
+      // operands are produced, the rest between the MFMAs, so that the requests reach
+      // the memory pipeline spread over the whole step
+      if (more) {
+#pragma unroll
+        for (int j = 0; j < kEarly; ++j)
+#pragma unroll
+          for (int t = 0; t < NT; ++t) b[kNext][t][j] = w_piece(kb + kWAhead, t, j);
+      }
+      float g[8];
+      unpack8(sgamma[kb * 16 + cg], g);
+#pragma unroll
+      for (int u = 0; u < RPT; ++u) {
+        float a[8], z[8], back[8], lo[8];
+        unpack8(xr[kb][u], a);
+        ss[u] += (double)sumsq8(xr[kb][u]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) z[i] = a[i] * g[i];
+        const uint4 hi = pack8_bf16(z);
+        unpack8(hi, back);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) lo[i] = z[i] - back[i];
+        const int slot = ahalf * 32 + ((RPT * rg + u) ^ aj);
+        sh.a[buf][0][aj][slot] = hi;
+        sh.a[buf][1][aj][slot] = pack8_bf16(lo);
+      }
+      if (kb + kAhead < KB && kb + kAhead < kblocks) fetch_x(kb + kAhead, xr[kb + kAhead]);
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (more && j + kEarly < 8) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) b[kNext][t][j + kEarly] = w_piece(kb + kWAhead, t, j + kEarly);
+        }
+        const int slot = half * 32 + (arow ^ j);
+        const bf16x8_t ahi = __builtin_bit_cast(bf16x8_t, sh.a[buf][0][j][slot]);
+        const bf16x8_t alo = __builtin_bit_cast(bf16x8_t, sh.a[buf][1][j][slot]);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, b[kb % WDEPTH][t][j]);
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi, bw, acc[t], 0, 0, 0);
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo, bw, acc[t], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- statistic
+  float rs[RPT];
+#pragma unroll
+  for (int u = 0; u < RPT; ++u) {
+    rs[u] = 1.0f / sqrtf((float)row16_sum_d(ss[u]) / (float)K + eps);
+    if (cg == 0) {
+      sh.rstd[RPT * rg + u] = rs[u];
+      rstd_out[row0 + RPT * rg + u] = rs[u];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int col = (wave * NT + t) * 32 + arow;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = (v / 4) * 8 + half * 4 + (v % 4);
+      logits[(row0 + row) * N + col] = acc[t][v] * sh.rstd[row];
+    }
+  }
+
+  // ---- sweep 2
+  uint16_t* yrow = y + (row0 + RPT * rg) * K + cg * 8;
+  uint8_t* qrow = q + (row0 + RPT * rg) * K + cg * 8;
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    if (kb < kblocks) {
+      float g[8];
+      unpack8(sgamma[kb * 16 + cg], g);
+#pragma unroll
+      for (int u = 0; u < RPT; ++u) {
+        float a[8], yv[8], qv[8];
+        unpack8(xr[kb][u], a);
+        float m = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          yv[i] = (a[i] * rs[u]) * g[i];
+          m = fmaxf(m, fabsf(yv[i]));
+        }
+        m = row16_max(m);
+        const float sc = make_scale<KIND, ROUND>(m);
+        const Divisor d = make_divisor(sc);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qv[i] = div_by_scale<ROUND>(yv[i], d);
+        *(uint4*)(yrow + (int64_t)u * K + kb * kGroup) = pack8_bf16(yv);
+        uint2 pk;
+        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+        *(uint2*)(qrow + (int64_t)u * K + kb * kGroup) = pk;
+        if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
+      }
+    }
+  }
+}
+
 hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, void* wpacked, void* y,
                                        float* rstd, float* logits, void* q, float* s, int64_t M, int K, int N,
                                        float eps, int round_scale, int kind, hipStream_t stream) {
@@ -253,26 +434,39 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
   }
   const dim3 grid((unsigned)(M / kRouterRows));
   const int tiles = N / 32;
-  // 8 waves when the column tiles split evenly over them (N = 256, 512), else 4
-#define FQ_ROUTER_GO(KINDV, ROUNDV, TPWV, WAVESV)                                                               \
-  hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, TPWV, WAVESV>), grid, dim3(64 * WAVESV), 0,    \
-                     stream, (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)wpacked, (uint16_t*)y,   \
-                     rstd, logits, (uint8_t*)q, s, M, K, N, eps)
-#define FQ_ROUTER_KIND(TPWV, WAVESV)                                                                            \
+  // 8 waves when the column tiles split evenly over them (N = 256, 512), else 4;
+  // rows held in registers when they fit beside the operands: K <= 2048 and one
+  // column tile per wave (N = 128, 256); streamed twice otherwise
+  constexpr int kResidentBlocks = 16;
+  const bool resident = K <= kResidentBlocks * kGroup;
+#define FQ_ROUTER_ARGS(WAVESV)                                                                                  \
+  grid, dim3(64 * WAVESV), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)wpacked,        \
+      (uint16_t*)y, rstd, logits, (uint8_t*)q, s, M, K, N, eps
+#define FQ_ROUTER_STREAMED(KINDV, ROUNDV, TPWV, WAVESV)                                                         \
+  hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, TPWV, WAVESV>), FQ_ROUTER_ARGS(WAVESV))
+#define FQ_ROUTER_RESIDENT(KINDV, ROUNDV, TPWV, WAVESV)                                                         \
+  if (resident)                                                                                                 \
+    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, kResidentBlocks, 2>), \
+                       FQ_ROUTER_ARGS(WAVESV));                                                                 \
+  else                                                                                                          \
+    FQ_ROUTER_STREAMED(KINDV, ROUNDV, TPWV, WAVESV)
+#define FQ_ROUTER_KIND(GO, TPWV, WAVESV)                                                                        \
   if (kind == kE5M2) {                                                                                          \
-    if (round_scale) FQ_ROUTER_GO(kE5M2, true, TPWV, WAVESV); else FQ_ROUTER_GO(kE5M2, false, TPWV, WAVESV);    \
+    if (round_scale) { GO(kE5M2, true, TPWV, WAVESV); } else { GO(kE5M2, false, TPWV, WAVESV); }                \
   } else {                                                                                                      \
-    if (round_scale) FQ_ROUTER_GO(kE4M3, true, TPWV, WAVESV); else FQ_ROUTER_GO(kE4M3, false, TPWV, WAVESV);    \
+    if (round_scale) { GO(kE4M3, true, TPWV, WAVESV); } else { GO(kE4M3, false, TPWV, WAVESV); }                \
   }
   switch (tiles) {
-    case 4: FQ_ROUTER_KIND(1, 4) break;
-    case 8: FQ_ROUTER_KIND(1, 8) break;
-    case 12: FQ_ROUTER_KIND(3, 4) break;
-    case 16: FQ_ROUTER_KIND(2, 8) break;
+    case 4: FQ_ROUTER_KIND(FQ_ROUTER_RESIDENT, 1, 4) break;
+    case 8: FQ_ROUTER_KIND(FQ_ROUTER_RESIDENT, 1, 8) break;
+    case 12: FQ_ROUTER_KIND(FQ_ROUTER_STREAMED, 3, 4) break;
+    case 16: FQ_ROUTER_KIND(FQ_ROUTER_STREAMED, 2, 8) break;
     default: return hipErrorInvalidValue;
   }
 #undef FQ_ROUTER_KIND
-#undef FQ_ROUTER_GO
+#undef FQ_ROUTER_RESIDENT
+#undef FQ_ROUTER_STREAMED
+#undef FQ_ROUTER_ARGS
   return hipGetLastError();
 }
 
