@@ -245,7 +245,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
 }
 
 
-// The same operation for K <= 128 * KB with the workgroup's rows of x held in
+// The same operation for K == 128 * KB with the workgroup's rows of x held in
 // registers, so that x is read from memory once and the GEMM does not wait for the
 // statistic.  rstd is a per-row factor of y, hence of the logits:
 //   logits[r, :] = rstd[r] * sum_k (x[r,k] * gamma[k]) * W[:, k]
@@ -271,7 +271,6 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
   constexpr int NT = TPW;
   constexpr int RPT = 8 / WAVES;
   constexpr int kAhead = 6;  // k blocks of x in flight ahead of the one worked on
-  constexpr int kEarly = 0;  // W pieces requested ahead of the MFMA loop rather than inside it
   constexpr int kWAhead = WDEPTH - 1;  // k blocks of W in flight ahead of the one worked on
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
@@ -280,7 +279,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
   const int ahalf = cg >> 3;
   const int arow = lane & 31;
   const int half = lane >> 5;
-  const int kblocks = K / kGroup;
+  constexpr int kblocks = KB;  // a constant trip count lets the compiler schedule across blocks
 
   floatx16_t acc[NT];
 #pragma unroll
@@ -308,62 +307,61 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
     }
 #pragma unroll
   for (int d = 0; d < kAhead; ++d)
-    if (d < KB && d < kblocks) fetch_x(d, xr[d]);
+    if (d < kblocks) fetch_x(d, xr[d]);
   for (int p = threadIdx.x; p < kblocks * 16; p += 64 * WAVES) sgamma[p] = *(const uint4*)(gamma + p * 8);
   __syncthreads();
 
-  // ---- sweep 1
+  // ---- sweep 1, software pipelined: the A operands of block kb + 1 are produced
+  // while the matrix cores work on block kb (double-buffered in LDS, one barrier
+  // per block)
+  auto produce = [&](int kb, const uint4 (&xk)[RPT]) {
+    float g[8];
+    unpack8(sgamma[kb * 16 + cg], g);
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb) {
-    if (kb < kblocks) {
-      const int buf = kb & 1;
-      const bool more = kb + kWAhead < kblocks;
-      const int kNext = (kb + kWAhead) % WDEPTH;
-      // the next block's W: the first kEarly pieces are requested before this block's
-      // operands are produced, the rest between the MFMAs, so that the requests reach
-      // the memory pipeline spread over the whole step
+    for (int u = 0; u < RPT; ++u) {
+      float a[8], z[8], back[8], lo[8];
+      unpack8(xk[u], a);
+      ss[u] += (double)sumsq8(xk[u]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) z[i] = a[i] * g[i];
+      const uint4 hi = pack8_bf16(z);
+      unpack8(hi, back);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) lo[i] = z[i] - back[i];
+      const int slot = ahalf * 32 + ((RPT * rg + u) ^ aj);
+      sh.a[kb & 1][0][aj][slot] = hi;
+      sh.a[kb & 1][1][aj][slot] = pack8_bf16(lo);
+    }
+  };
+  produce(0, xr[0]);
+  if (kAhead < kblocks) fetch_x(kAhead, xr[kAhead]);
+  __syncthreads();
+#pragma unroll
+  for (int kb = 0; kb < kblocks; ++kb) {
+    const int buf = kb & 1;
+    const bool more = kb + kWAhead < kblocks;
+    const int kNext = (kb + kWAhead) % WDEPTH;
+    if (kb + 1 < kblocks) {
+      produce(kb + 1, xr[kb + 1]);
+      if (kb + 1 + kAhead < kblocks) fetch_x(kb + 1 + kAhead, xr[kb + 1 + kAhead]);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
       if (more) {
 #pragma unroll
-        for (int j = 0; j < kEarly; ++j)
-#pragma unroll
-          for (int t = 0; t < NT; ++t) b[kNext][t][j] = w_piece(kb + kWAhead, t, j);
+        for (int t = 0; t < NT; ++t) b[kNext][t][j] = w_piece(kb + kWAhead, t, j);
       }
-      float g[8];
-      unpack8(sgamma[kb * 16 + cg], g);
+      const int slot = half * 32 + (arow ^ j);
+      const bf16x8_t ahi = __builtin_bit_cast(bf16x8_t, sh.a[buf][0][j][slot]);
+      const bf16x8_t alo = __builtin_bit_cast(bf16x8_t, sh.a[buf][1][j][slot]);
 #pragma unroll
-      for (int u = 0; u < RPT; ++u) {
-        float a[8], z[8], back[8], lo[8];
-        unpack8(xr[kb][u], a);
-        ss[u] += (double)sumsq8(xr[kb][u]);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) z[i] = a[i] * g[i];
-        const uint4 hi = pack8_bf16(z);
-        unpack8(hi, back);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) lo[i] = z[i] - back[i];
-        const int slot = ahalf * 32 + ((RPT * rg + u) ^ aj);
-        sh.a[buf][0][aj][slot] = hi;
-        sh.a[buf][1][aj][slot] = pack8_bf16(lo);
-      }
-      if (kb + kAhead < KB && kb + kAhead < kblocks) fetch_x(kb + kAhead, xr[kb + kAhead]);
-      __syncthreads();
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        if (more && j + kEarly < 8) {
-#pragma unroll
-          for (int t = 0; t < NT; ++t) b[kNext][t][j + kEarly] = w_piece(kb + kWAhead, t, j + kEarly);
-        }
-        const int slot = half * 32 + (arow ^ j);
-        const bf16x8_t ahi = __builtin_bit_cast(bf16x8_t, sh.a[buf][0][j][slot]);
-        const bf16x8_t alo = __builtin_bit_cast(bf16x8_t, sh.a[buf][1][j][slot]);
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, b[kb % WDEPTH][t][j]);
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi, bw, acc[t], 0, 0, 0);
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo, bw, acc[t], 0, 0, 0);
-        }
+      for (int t = 0; t < NT; ++t) {
+        const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, b[kb % WDEPTH][t][j]);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi, bw, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo, bw, acc[t], 0, 0, 0);
       }
     }
+    __syncthreads();
   }
 
   // ---- statistic
@@ -391,8 +389,8 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
   uint16_t* yrow = y + (row0 + RPT * rg) * K + cg * 8;
   uint8_t* qrow = q + (row0 + RPT * rg) * K + cg * 8;
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb) {
-    if (kb < kblocks) {
+  for (int kb = 0; kb < kblocks; ++kb) {
+    {
       float g[8];
       unpack8(sgamma[kb * 16 + cg], g);
 #pragma unroll
@@ -435,18 +433,20 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
   const dim3 grid((unsigned)(M / kRouterRows));
   const int tiles = N / 32;
   // 8 waves when the column tiles split evenly over them (N = 256, 512), else 4;
-  // rows held in registers when they fit beside the operands: K <= 2048 and one
-  // column tile per wave (N = 128, 256); streamed twice otherwise
-  constexpr int kResidentBlocks = 16;
-  const bool resident = K <= kResidentBlocks * kGroup;
+  // rows held in registers when they fit beside the operands and K is one of the
+  // instantiated widths: one column tile per wave (N = 128, 256), K = 1024 or 2048;
+  // streamed twice otherwise
 #define FQ_ROUTER_ARGS(WAVESV)                                                                                  \
   grid, dim3(64 * WAVESV), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)wpacked,        \
       (uint16_t*)y, rstd, logits, (uint8_t*)q, s, M, K, N, eps
 #define FQ_ROUTER_STREAMED(KINDV, ROUNDV, TPWV, WAVESV)                                                         \
   hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, TPWV, WAVESV>), FQ_ROUTER_ARGS(WAVESV))
 #define FQ_ROUTER_RESIDENT(KINDV, ROUNDV, TPWV, WAVESV)                                                         \
-  if (resident)                                                                                                 \
-    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, kResidentBlocks, 2>), \
+  if (K == 2048)                                                                                                \
+    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, 16, 2>),              \
+                       FQ_ROUTER_ARGS(WAVESV));                                                                 \
+  else if (K == 1024)                                                                                           \
+    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, 8, 2>),               \
                        FQ_ROUTER_ARGS(WAVESV));                                                                 \
   else                                                                                                          \
     FQ_ROUTER_STREAMED(KINDV, ROUNDV, TPWV, WAVESV)

@@ -447,7 +447,8 @@ def test_block_quant(gpu, M, N, round_scale):
 
 
 # ------------------------------------------------------------------ RMSNorm + router GEMM + quant
-@pytest.mark.parametrize("M,N,K", [(8192, 256, 2048), (256, 128, 1536), (128, 512, 4096), (384, 384, 7168)])
+@pytest.mark.parametrize("M,N,K", [(8192, 256, 2048), (256, 128, 1536), (128, 512, 4096), (384, 384, 7168),
+                                   (256, 128, 1024), (128, 256, 1024), (128, 128, 2048)])
 @pytest.mark.parametrize("round_scale", [False, True])
 def test_rms_norm_fp32_gemm_block_quant(gpu, M, N, K, round_scale):
     """reference tests/test_norm.py:251-287 (x = randn**2, weights randn)."""
