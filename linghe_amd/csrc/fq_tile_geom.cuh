@@ -102,7 +102,8 @@ __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int 
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
   // base is the same for the whole workgroup (scalar registers); a tile spans at
-  // most 128 rows of at most 32 KB, so lane offsets fit 32 bits
+  // most 128 rows of at most 2^24 bytes (the widest input the entry points accept),
+  // so lane offsets fit 32 bits
   const uint8_t* b = (const uint8_t*)base;
   const uint32_t pitch = (uint32_t)ld * 2u;
   const uint32_t off0 = (uint32_t)(rg * RPT) * pitch + (uint32_t)cg * 16u;
