@@ -94,12 +94,12 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
 // SwiGLU forward + quant.  y = (sigmoid(x1)*x1)*x2 [*w_row]   (fp32)
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED>
-__global__ __launch_bounds__(256) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
+__global__ __launch_bounds__(512) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {
-  constexpr int RPT = 8;
+  constexpr int RPT = 4;
   __shared__ TileShared<RPT> sh;
   __shared__ ExpertScanShared scan;
-  const TileGeom g = resolve_tile<BATCHED, 256>(M, n / kGroup, n, batch, scan);
+  const TileGeom g = resolve_tile<BATCHED, 512>(M, n / kGroup, n, batch, scan);
   if (!g.valid) return;
   const int64_t ld = 2 * (int64_t)n;
   uint4 r1[RPT], r2[RPT];
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void silu_quant_fwd_kernel(const uint16_t* __r
 // evaluated in the order fp32 autograd evaluates them.
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, bool BATCHED>
-__global__ __launch_bounds__(512) void silu_quant_bwd_kernel(const uint16_t* __restrict__ gr,
+__global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* __restrict__ gr,
                                                              const uint16_t* __restrict__ x, RowWeight weight,
                                                              OutPtrs out, float* __restrict__ dw_part, int64_t M,
                                                              int n, BatchArgs batch) {
@@ -221,15 +221,15 @@ __global__ __launch_bounds__(256) void rowsum_kernel(const float* __restrict__ p
 //   y = (x * rstd[row]) * gamma[col]
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, int MODE>
-__global__ __launch_bounds__(256) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
+__global__ __launch_bounds__(512) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
                                                                  const uint16_t* __restrict__ gamma,
                                                                  const float* __restrict__ rstd, OutPtrs out,
                                                                  int64_t M, int n) {
-  constexpr int RPT = 8;
+  constexpr int RPT = 4;
   __shared__ TileShared<RPT> sh;
   __shared__ ExpertScanShared scan;
   BatchArgs none{nullptr, 0, 0};
-  const TileGeom g = resolve_tile<false, 256>(M, n / kGroup, n, none, scan);
+  const TileGeom g = resolve_tile<false, 512>(M, n / kGroup, n, none, scan);
   if (!g.valid) return;
   uint4 raw[RPT];
   load_rows<RPT>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
@@ -296,7 +296,7 @@ hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_b
   RowWeight w{weight, weight_bf16};
   const int64_t tiles = row_blocks * (n / kGroup);
   if (tiles == 0) return hipSuccess;
-  const dim3 grid((unsigned)tiles), block(256);
+  const dim3 grid((unsigned)tiles), block(512);
   const bool batched = counts != nullptr;
   const bool weighted = weight != nullptr;
   FQ_DISPATCH_KIND(kind, K,
@@ -342,7 +342,7 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
   const int64_t tiles = ((M + kGroup - 1) / kGroup) * (n / kGroup);
   if (tiles == 0) return hipSuccess;
-  const dim3 grid((unsigned)tiles), block(256);
+  const dim3 grid((unsigned)tiles), block(512);
   FQ_DISPATCH_KIND(kind, K,
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
