@@ -107,7 +107,7 @@ __device__ __forceinline__ double sumsq(const uint4 (&raw)[NCHUNK]) {
 }
 
 // ---------------------------------------------------------------------------
-// forward: OUT = 0 -> bf16 y ; 1 -> fp8 codes + [nb, M] scales ; 2 -> rstd only
+// forward: OUT = 0 -> bf16 y ; 1 -> fp8 codes + [nb, M] scales
 // ---------------------------------------------------------------------------
 template <int T, int NCHUNK, bool REUSE, int OUT, int KIND, bool ROUND>
 __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restrict__ x,
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
   __shared__ RowShared<T> sh;
   const int tid = threadIdx.x;
   uint4 gm[NCHUNK];
-  if constexpr (OUT != 2) load_row<T, NCHUNK>(gamma, n, gm);
+  load_row<T, NCHUNK>(gamma, n, gm);
   const int64_t G = gridDim.x;  // rows blockIdx.x, +G, +2G, ...
   const int64_t r0 = blockIdx.x;
   const int64_t r1 = M;
@@ -135,7 +135,6 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
       r = rstd_from_sumsq((float)ss, n, eps);
       if (tid == 0) rstd[row] = r;
     }
-    if constexpr (OUT == 2) return;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
       const int c = tid + k * T;
@@ -176,6 +175,35 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
       if (row + 2 * G < r1) load_row<T, NCHUNK>(x + (row + 2 * G) * n, n, bufA);
       process(bufB, row + G, 1);
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// statistic only (the first pass of RMSNorm + quant, output_mode 2): one wave per
+// row, eight 16-byte loads per lane in flight, nothing kept.  Few registers, so a
+// CU holds its 32 waves and a 16384-row input is two rows per wave with no tail.
+// Same arithmetic as everywhere else: 8-element group sums added in double.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict__ x, float* __restrict__ rstd,
+                                                     int64_t M, int n, float eps) {
+  const int lane = threadIdx.x;
+  const int chunks = n >> 3;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint4* p = (const uint4*)(x + row * n);
+    double ss = 0.0;
+    for (int c0 = 0; c0 < chunks; c0 += 512) {
+      uint4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int c = c0 + u * 64 + lane;
+        v[u] = make_uint4(0, 0, 0, 0);
+        if (c < chunks) v[u] = p[c];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ss += (double)sumsq8(v[u]);
+    }
+    ss = wave_sum_d(ss);
+    if (lane == 0) rstd[row] = rstd_from_sumsq((float)ss, n, eps);
   }
 }
 
@@ -385,9 +413,9 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
   FQ_FWD_SHAPES(hipLaunchKernelGGL((rmsnorm_fwd_kernel<kT, kNC, REUSE, QUANT, KINDV, ROUNDV>), grid,       \
                                    dim3(kT), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, out,   \
                                    scale, rstd, M, n, eps, rows_per_wg);)
-  // quant: 0 = bf16 output, 1 = fp8 codes + scales, 2 = statistic only
+  // quant: 0 = bf16 output, 1 = fp8 codes + scales, 2 = statistic only (its own kernel)
   if (quant == 2) {
-    FQ_LAUNCH_FWD(false, 2, kE4M3, false)
+    hipLaunchKernelGGL(rowstat_kernel, grid, dim3(64), 0, stream, (const uint16_t*)x, rstd, M, n, eps);
   } else if (!quant) {
     if (reuse_rstd) { FQ_LAUNCH_FWD(true, 0, kE4M3, false) } else { FQ_LAUNCH_FWD(false, 0, kE4M3, false) }
   } else if (kind == kE5M2) {
