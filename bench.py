@@ -29,7 +29,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-SINGLE_PASS_CASES = {"cfg1_single"}  # RMSNorm+quant mode 2 with the workspace (one pass over x)
+SINGLE_PASS_CASES = {"cfg1_single", "cfg5b_single"}  # RMSNorm+quant mode 2 with the workspace (one pass over x)
 INFINITY_CACHE_BYTES = 256 << 20
 FP8 = torch.float8_e4m3fn
 
@@ -113,6 +113,7 @@ def build_cases(names, dev):
     add("cfg1", build=lambda: rms_quant_case("cfg1", configs.cfg1_rmsnorm_quant(), 2))
     add("cfg1_single", build=lambda: rms_quant_case("cfg1_single", configs.cfg1_rmsnorm_quant(), 2))
     add("cfg5b", build=lambda: rms_quant_case("cfg5b", cfg5(), 2))
+    add("cfg5b_single", build=lambda: rms_quant_case("cfg5b_single", cfg5(), 2))
     add("cfg5c", build=lambda: rms_quant_case("cfg5c", cfg5(), 1))
 
     # ---------------------------------------------------------------- cfg2
@@ -458,7 +459,8 @@ def time_cpu(case, budget_s):
 # the difference is the second read of x.
 CFG1_MEASURED_TRAFFIC_BYTES = 102.48e6
 
-ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c", "next_permute",
+ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5b_single", "cfg5c",
+       "next_permute",
        "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router"]
 
 

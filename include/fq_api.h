@@ -123,11 +123,13 @@ int64_t fq_rmsnorm_quant_workspace_bytes(int64_t M, int64_t n);
  * statistic through it, every entry stamped with a per-call counter, so the
  * buffer needs no clearing between calls and can be shared by calls of any
  * shape on one stream (calls that may overlap in time need a buffer each; clear
- * it again after 2^32 calls).  Without it, for problems of more than 1024
- * tiles of 128x128 (the single pass pays only while every tile is resident on
- * the GPU at once), or while `stream` is being captured into a graph (a replay
- * would repeat the stamp), mode 2 runs as two passes - the row statistic, then
- * the tile kernel - and reads x twice. */
+ * it again after 2^32 calls).  The workgroups of the single pass wait for each
+ * other, so it wants the GPU to itself; every wait is bounded
+ * (fq_set_wait_limit) and a workgroup that gives up recomputes what it waited
+ * for, so results never depend on timing.  Without a workspace, or while
+ * `stream` is being captured into a graph (a replay would repeat the stamp),
+ * mode 2 runs as two passes - the row statistic, then the tile kernel - and
+ * reads x twice; that is the faster variant at every size measured so far. */
 int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt, float* st,
                          int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
                          void* workspace, int64_t workspace_bytes, void* stream);

@@ -207,10 +207,8 @@ int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, fl
   FQ_REQUIRE(aligned16(x) && aligned16(gamma), FQ_ERR_ARG, "%s: misaligned pointer", fn);
   hipStream_t st_ = (hipStream_t)stream;
   if ((rc = check_tiles(fn, ((M + 127) / 128) * (n / 128)))) return rc;
-  // The single-pass kernel keeps every tile in registers while its slab's statistic
-  // is assembled; that pays only while the whole grid is resident at once (4
-  // workgroups on each of the 256 CUs).  Larger problems run as two passes.
-  bool single_pass = output_mode == 2 && workspace != nullptr && ((M + 127) / 128) * (n / 128) <= 1024;
+  // single pass only when the caller brings the exchange workspace
+  bool single_pass = output_mode == 2 && workspace != nullptr;
   if (single_pass) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st_, &cap) != hipSuccess) {

@@ -16,9 +16,9 @@ _MAX_HIDDEN = 8192  # the reference asserts next_power_of_2(n) <= 8192
 # output_mode 2 of triton_rms_norm_and_block_quant_forward:
 #   False  two passes (row statistic, then the tile kernel): the fastest measured
 #          variant on MI355X at every size tried;
-#   True   hand the library its workspace, so that problems of at most 1024 tiles
-#          run as ONE pass over x (the statistic is exchanged between workgroups
-#          inside the kernel): algorithmic HBM traffic, ~8 % slower at 8192x2048.
+#   True   hand the library its workspace, so that the call is ONE pass over x (the
+#          statistic is exchanged between workgroups inside the kernel):
+#          algorithmic HBM traffic, 20-25 % slower at the sizes measured.
 SINGLE_PASS = False
 
 
