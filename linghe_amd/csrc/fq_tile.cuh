@@ -153,7 +153,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
       pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
       const int i = rg * RPT + s;
-      // scalar tile base + 32-bit lane offset (128 rows of at most 16 KB)
+      // scalar tile base + 32-bit lane offset (128 rows of at most 2^23 bytes)
       if (FULL || i < o.rows_valid) *(uint2*)((o.q + o.q_off) + ((uint32_t)i * (uint32_t)o.q_ld + (uint32_t)cg * 8u)) = pk;
     }
   }
