@@ -188,7 +188,12 @@ __global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict_
                                                      int64_t M, int n, float eps) {
   const int lane = threadIdx.x;
   const int chunks = n >> 3;
-  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+  // Rows are taken from the END of the matrix backwards.  The tile kernel that follows
+  // walks the matrix forwards, so it starts with the rows this kernel read last, which
+  // are the ones still in the last-level cache: for an input about the size of that
+  // cache roughly half of the second read never reaches HBM.
+  for (int64_t k = blockIdx.x; k < M; k += gridDim.x) {
+    const int64_t row = M - 1 - k;
     const uint4* p = (const uint4*)(x + row * n);
     double ss = 0.0;
     for (int c0 = 0; c0 < chunks; c0 += 512) {
