@@ -291,6 +291,44 @@ def test_rmsnorm_quant_single_pass_wait_bound(gpu):
     check_quant_pair("rms.two_pass.col", ref[3], ref[4], qt, st, **EXACT)
 
 
+@pytest.mark.parametrize("M,N", [(8192, 2048), (4096 + 40, 7168), (16384, 512), (3000, 1536)])
+@pytest.mark.parametrize("short_wait", [False, True])
+def test_rmsnorm_quant_single_pass_many_steps(gpu, M, N, short_wait):
+    """Shapes with more tiles than the device holds workgroups: every workgroup of
+    the single-pass kernel walks several tiles.  Its outputs, statistic included,
+    must equal the two-pass path bit for bit (both add the same exact group sums),
+    also when every wait is cut to one poll and the workgroups fall back to
+    recomputing the statistic in the middle of their sequence."""
+    from linghe_amd import _lib
+    from linghe_amd.utils.norm import triton_rms_norm_and_block_quant_forward as fwd
+    import linghe_amd.utils.norm as norm_mod
+
+    announce("rmsnorm+quant single pass, many steps", M, N, short_wait)
+    g = gen(29)
+    x = randn_bf16(g, M, N, scale=2.0)
+    w = gamma_bf16(g, N)
+    xd, wd = _dev(x, gpu), _dev(w, gpu)
+    two = fwd(xd, wd, round_scale=False, output_mode=2)
+    torch.cuda.synchronize()
+    norm_mod.SINGLE_PASS = True
+    try:
+        if short_wait:
+            _lib.lib.fq_set_wait_limit(1)
+        one = fwd(xd, wd, round_scale=False, output_mode=2)
+        again = fwd(xd, wd, round_scale=False, output_mode=2)
+        torch.cuda.synchronize()
+    finally:
+        _lib.lib.fq_set_wait_limit(0)
+        norm_mod.SINGLE_PASS = False
+    names = ("q", "s", "rstd", "qt", "st")
+    for name, a, b, c in zip(names, two, one, again):
+        av, bv, cv = (t.view(torch.uint8).cpu() for t in (a, b, c))
+        assert torch.equal(av, bv), f"{name}: single pass differs from two passes"
+        assert torch.equal(bv, cv), f"{name}: second single-pass call differs"
+    ref = O.rms_norm_and_block_quant_forward(x[:256], w, rstd=one[2][:256].cpu())
+    check_quant_pair("rms.single.steps.row", ref[0], ref[1], one[0][:256], one[1][:, :256], **EXACT)
+
+
 # ------------------------------------------------------------------ SwiGLU
 @pytest.mark.parametrize("M,N,coef", [(2048, 1024, 1.0), (1024, 4096, 1.0), (1000, 1536, 1.0),
                                       (512, 1536 * 8, 100.0), (512, 1536 * 8, 0.0)])
