@@ -216,7 +216,7 @@ __global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict_
 // backward: dx = r*g*w - r^3 * x * sum(x*g*w)/n ; dgamma partial += x*g*r
 // ---------------------------------------------------------------------------
 template <int T, int NCHUNK, bool REUSE>
-__global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ dy,
+__global__ __launch_bounds__(T, T == 512 ? 4 : 1) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ dy,
                                                         const uint16_t* __restrict__ x,
                                                         const uint16_t* __restrict__ gamma,
                                                         const float* __restrict__ rstd_in,
@@ -280,7 +280,20 @@ __global__ __launch_bounds__(T) void rmsnorm_bwd_kernel(const uint16_t* __restri
     }
   };
 
-  if (r0 < r1) {  // the next row is prefetched into a second register set
+  if constexpr (T == 512) {
+    // wide rows: one row in registers (about 100 of them), so that two 512-thread
+    // workgroups fit a CU and cover each other's waits; prefetching the next row into a
+    // second register set costs that second workgroup and is slower (179 vs 155 us at
+    // 16384 x 7168)
+    uint4 xa[NCHUNK], ga[NCHUNK];
+    int parity = 0;
+    for (int64_t row = r0; row < r1; row += G) {
+      load_row<T, NCHUNK>(x + row * n, n, xa);
+      load_row<T, NCHUNK>(dy + row * n, n, ga);
+      process(xa, ga, row, parity);
+      parity ^= 1;
+    }
+  } else if (r0 < r1) {  // the next row is prefetched into a second register set
     uint4 xa[NCHUNK], ga[NCHUNK], xb[NCHUNK], gb[NCHUNK];
     load_row<T, NCHUNK>(x + r0 * n, n, xa);
     load_row<T, NCHUNK>(dy + r0 * n, n, ga);
@@ -384,7 +397,8 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __rest
 // ---------------------------------------------------------------------------
 // Forward kernels: one wave per row (64-thread workgroups, no barrier), every load
 // of a row in flight at once and the next row prefetched.
-// Backward kernel: 256 threads per row (it also carries the dgamma accumulators).
+// Backward kernel: 256 threads per row (it also carries the dgamma accumulators), 512
+// for rows wider than 4096.
 static void pick_row_shape(int n, int T, int& nchunk) {
   const int chunks = (n + 7) / 8;
   nchunk = (chunks + T - 1) / T;
@@ -399,9 +413,8 @@ static void pick_row_shape(int n, int T, int& nchunk) {
   FQ_ROW_CASE(64, 10, __VA_ARGS__) FQ_ROW_CASE(64, 11, __VA_ARGS__) FQ_ROW_CASE(64, 12, __VA_ARGS__) \
   FQ_ROW_CASE(64, 13, __VA_ARGS__) FQ_ROW_CASE(64, 14, __VA_ARGS__) FQ_ROW_CASE(64, 15, __VA_ARGS__) \
   FQ_ROW_CASE(64, 16, __VA_ARGS__) { return hipErrorInvalidValue; }
-#define FQ_BWD_SHAPES(...)                                                                           \
-  FQ_ROW_CASE(256, 1, __VA_ARGS__) FQ_ROW_CASE(256, 2, __VA_ARGS__) FQ_ROW_CASE(256, 3, __VA_ARGS__) \
-  FQ_ROW_CASE(256, 4, __VA_ARGS__) { return hipErrorInvalidValue; }
+#define FQ_BWD_SHAPES(...) \
+  FQ_ROW_CASE(256, 1, __VA_ARGS__) FQ_ROW_CASE(256, 2, __VA_ARGS__) { return hipErrorInvalidValue; }
 
 hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* scale, float* rstd, int64_t M,
                               int n, float eps, int reuse_rstd, int quant, int round_scale, int kind,
@@ -453,7 +466,14 @@ hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, 
   FQ_BWD_SHAPES(hipLaunchKernelGGL((rmsnorm_bwd_kernel<kT, kNC, REUSE>), grid, dim3(kT), 0, stream,        \
                                    (const uint16_t*)dy, (const uint16_t*)x, (const uint16_t*)gamma, rstd,  \
                                    (uint16_t*)dx, dg_part, M, n, eps, rows_per_wg);)
-  if (rstd) { FQ_LAUNCH_BWD(true) } else { FQ_LAUNCH_BWD(false) }
+#define FQ_LAUNCH_BWD_WIDE(REUSE)                                                                          \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<512, 2, REUSE>), grid, dim3(512), 0, stream, (const uint16_t*)dy, \
+                     (const uint16_t*)x, (const uint16_t*)gamma, rstd, (uint16_t*)dx, dg_part, M, n, eps,  \
+                     rows_per_wg)
+  if (nchunk > 2) {  // n > 4096: 512 threads x 2 chunks
+    if (rstd) { FQ_LAUNCH_BWD_WIDE(true); } else { FQ_LAUNCH_BWD_WIDE(false); }
+  } else if (rstd) { FQ_LAUNCH_BWD(true) } else { FQ_LAUNCH_BWD(false) }
+#undef FQ_LAUNCH_BWD_WIDE
 #undef FQ_LAUNCH_BWD
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
