@@ -216,7 +216,7 @@ __global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict_
 // backward: dx = r*g*w - r^3 * x * sum(x*g*w)/n ; dgamma partial += x*g*r
 // ---------------------------------------------------------------------------
 template <int T, int NCHUNK, bool REUSE>
-__global__ __launch_bounds__(T, T == 512 ? 4 : 1) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ dy,
+__global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ dy,
                                                         const uint16_t* __restrict__ x,
                                                         const uint16_t* __restrict__ gamma,
                                                         const float* __restrict__ rstd_in,
@@ -280,11 +280,11 @@ __global__ __launch_bounds__(T, T == 512 ? 4 : 1) void rmsnorm_bwd_kernel(const 
     }
   };
 
-  if constexpr (T == 512) {
-    // wide rows: one row in registers (about 100 of them), so that two 512-thread
-    // workgroups fit a CU and cover each other's waits; prefetching the next row into a
-    // second register set costs that second workgroup and is slower (179 vs 155 us at
-    // 16384 x 7168)
+  // One row in registers at a time (about 100 of them with two chunks per thread), so
+  // that two 512-thread workgroups fit a CU and cover each other's waits.  Prefetching
+  // the next row into a second register set costs that second workgroup and is slower
+  // (179 vs 155 us at 16384 x 7168).
+  {
     uint4 xa[NCHUNK], ga[NCHUNK];
     int parity = 0;
     for (int64_t row = r0; row < r1; row += G) {
@@ -292,24 +292,6 @@ __global__ __launch_bounds__(T, T == 512 ? 4 : 1) void rmsnorm_bwd_kernel(const 
       load_row<T, NCHUNK>(dy + row * n, n, ga);
       process(xa, ga, row, parity);
       parity ^= 1;
-    }
-  } else if (r0 < r1) {  // the next row is prefetched into a second register set
-    uint4 xa[NCHUNK], ga[NCHUNK], xb[NCHUNK], gb[NCHUNK];
-    load_row<T, NCHUNK>(x + r0 * n, n, xa);
-    load_row<T, NCHUNK>(dy + r0 * n, n, ga);
-    for (int64_t row = r0; row < r1; row += 2 * G) {
-      if (row + G < r1) {
-        load_row<T, NCHUNK>(x + (row + G) * n, n, xb);
-        load_row<T, NCHUNK>(dy + (row + G) * n, n, gb);
-      }
-      process(xa, ga, row, 0);
-      if (row + G < r1) {
-        if (row + 2 * G < r1) {
-          load_row<T, NCHUNK>(x + (row + 2 * G) * n, n, xa);
-          load_row<T, NCHUNK>(dy + (row + 2 * G) * n, n, ga);
-        }
-        process(xb, gb, row + G, 1);
-      }
     }
   }
   // every workgroup writes its (possibly zero) partial: the reduction reads all of them
@@ -320,6 +302,110 @@ __global__ __launch_bounds__(T, T == 512 ? 4 : 1) void rmsnorm_bwd_kernel(const 
       float4* dst = (float4*)(dg_part + (int64_t)blockIdx.x * n + c * 8);
       dst[0] = make_float4(acc[k][0], acc[k][1], acc[k][2], acc[k][3]);
       dst[1] = make_float4(acc[k][4], acc[k][5], acc[k][6], acc[k][7]);
+    }
+  }
+}
+
+// Backward for narrow rows (n <= 2048): one wave per row, so the two row sums are
+// wave reductions and no barrier or LDS traffic sits between a row's loads and its
+// stores.  The four waves of a workgroup walk their own rows and keep their own
+// dgamma accumulators, added in wave order at the end: one partial row per workgroup
+// as in the kernel above.  Lane l holds the 16-byte chunks l, l+64, ...
+template <int NCHUNK, bool REUSE>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_wave_kernel(const uint16_t* __restrict__ dy,
+                                                               const uint16_t* __restrict__ x,
+                                                               const uint16_t* __restrict__ gamma,
+                                                               const float* __restrict__ rstd_in,
+                                                               uint16_t* __restrict__ dx,
+                                                               float* __restrict__ dg_part, int64_t M, int n,
+                                                               float eps) {
+  __shared__ float4 combine[3][NCHUNK * 2][64];  // waves 1..3: [chunk half][lane]
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int chunks = n >> 3;
+  uint4 gm[NCHUNK];
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) {
+    const int c = lane + k * 64;
+    gm[k] = make_uint4(0, 0, 0, 0);
+    if (c < chunks) gm[k] = *(const uint4*)(gamma + c * 8);
+  }
+  float acc[NCHUNK][8];
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[k][j] = 0.f;
+
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < M; row += stride) {
+    uint4 rx[NCHUNK], rg[NCHUNK];
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      const int c = lane + k * 64;
+      rx[k] = make_uint4(0, 0, 0, 0);
+      rg[k] = make_uint4(0, 0, 0, 0);
+      if (c < chunks) {
+        rx[k] = *(const uint4*)(x + row * n + c * 8);
+        rg[k] = *(const uint4*)(dy + row * n + c * 8);
+      }
+    }
+    float dot = 0.f;
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      float a[8], g[8], w[8];
+      unpack8(rx[k], a);
+      unpack8(rg[k], g);
+      unpack8(gm[k], w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
+    }
+    dot = wave_sum(dot);
+    float r;
+    if constexpr (REUSE) {
+      r = rstd_in[row];
+    } else {
+      r = rstd_from_sumsq((float)wave_sum_d(sumsq<NCHUNK>(rx)), n, eps);
+    }
+    const float coef = ((r * r) * r) * dot / (float)n;
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      const int c = lane + k * 64;
+      float a[8], g[8], w[8], o[8];
+      unpack8(rx[k], a);
+      unpack8(rg[k], g);
+      unpack8(gm[k], w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        o[j] = (r * g[j]) * w[j] - coef * a[j];
+        acc[k][j] += (a[j] * g[j]) * r;
+      }
+      if (c < chunks) *(uint4*)(dx + row * n + c * 8) = pack8_bf16(o);
+    }
+  }
+  // waves 1..3 hand their accumulators to wave 0, which adds them in wave order
+  if (wave > 0) {
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      combine[wave - 1][2 * k][lane] = make_float4(acc[k][0], acc[k][1], acc[k][2], acc[k][3]);
+      combine[wave - 1][2 * k + 1][lane] = make_float4(acc[k][4], acc[k][5], acc[k][6], acc[k][7]);
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+#pragma unroll
+      for (int w = 0; w < 3; ++w) {
+        const float4 lo = combine[w][2 * k][lane], hi = combine[w][2 * k + 1][lane];
+        acc[k][0] += lo.x; acc[k][1] += lo.y; acc[k][2] += lo.z; acc[k][3] += lo.w;
+        acc[k][4] += hi.x; acc[k][5] += hi.y; acc[k][6] += hi.z; acc[k][7] += hi.w;
+      }
+      const int c = lane + k * 64;
+      if (c < chunks) {
+        float4* dst = (float4*)(dg_part + (int64_t)blockIdx.x * n + c * 8);
+        dst[0] = make_float4(acc[k][0], acc[k][1], acc[k][2], acc[k][3]);
+        dst[1] = make_float4(acc[k][4], acc[k][5], acc[k][6], acc[k][7]);
+      }
     }
   }
 }
@@ -397,8 +483,8 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __rest
 // ---------------------------------------------------------------------------
 // Forward kernels: one wave per row (64-thread workgroups, no barrier), every load
 // of a row in flight at once and the next row prefetched.
-// Backward kernel: 256 threads per row (it also carries the dgamma accumulators), 512
-// for rows wider than 4096.
+// Backward kernels: one wave per row up to n = 2048, 512 threads per row beyond (they
+// also carry the dgamma accumulators).
 static void pick_row_shape(int n, int T, int& nchunk) {
   const int chunks = (n + 7) / 8;
   nchunk = (chunks + T - 1) / T;
@@ -413,8 +499,6 @@ static void pick_row_shape(int n, int T, int& nchunk) {
   FQ_ROW_CASE(64, 10, __VA_ARGS__) FQ_ROW_CASE(64, 11, __VA_ARGS__) FQ_ROW_CASE(64, 12, __VA_ARGS__) \
   FQ_ROW_CASE(64, 13, __VA_ARGS__) FQ_ROW_CASE(64, 14, __VA_ARGS__) FQ_ROW_CASE(64, 15, __VA_ARGS__) \
   FQ_ROW_CASE(64, 16, __VA_ARGS__) { return hipErrorInvalidValue; }
-#define FQ_BWD_SHAPES(...) \
-  FQ_ROW_CASE(256, 1, __VA_ARGS__) FQ_ROW_CASE(256, 2, __VA_ARGS__) { return hipErrorInvalidValue; }
 
 hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* scale, float* rstd, int64_t M,
                               int n, float eps, int reuse_rstd, int quant, int round_scale, int kind,
@@ -457,24 +541,32 @@ int64_t rmsnorm_bwd_partials(int64_t M) {
 hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
                               float* dgamma, float* dg_part, int64_t n_partials, int64_t M, int n, float eps,
                               hipStream_t stream) {
-  int nchunk;
-  pick_row_shape(n, 256, nchunk);
   const int64_t P = n_partials;
   const int rows_per_wg = (int)((M + P - 1) / P);
   const dim3 grid((unsigned)P);
-#define FQ_LAUNCH_BWD(REUSE)                                                                               \
-  FQ_BWD_SHAPES(hipLaunchKernelGGL((rmsnorm_bwd_kernel<kT, kNC, REUSE>), grid, dim3(kT), 0, stream,        \
-                                   (const uint16_t*)dy, (const uint16_t*)x, (const uint16_t*)gamma, rstd,  \
-                                   (uint16_t*)dx, dg_part, M, n, eps, rows_per_wg);)
-#define FQ_LAUNCH_BWD_WIDE(REUSE)                                                                          \
-  hipLaunchKernelGGL((rmsnorm_bwd_kernel<512, 2, REUSE>), grid, dim3(512), 0, stream, (const uint16_t*)dy, \
-                     (const uint16_t*)x, (const uint16_t*)gamma, rstd, (uint16_t*)dx, dg_part, M, n, eps,  \
+#define FQ_LAUNCH_BWD_BLOCK(NC, REUSE)                                                                      \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<512, NC, REUSE>), grid, dim3(512), 0, stream, (const uint16_t*)dy, \
+                     (const uint16_t*)x, (const uint16_t*)gamma, rstd, (uint16_t*)dx, dg_part, M, n, eps,   \
                      rows_per_wg)
-  if (nchunk > 2) {  // n > 4096: 512 threads x 2 chunks
-    if (rstd) { FQ_LAUNCH_BWD_WIDE(true); } else { FQ_LAUNCH_BWD_WIDE(false); }
-  } else if (rstd) { FQ_LAUNCH_BWD(true) } else { FQ_LAUNCH_BWD(false) }
-#undef FQ_LAUNCH_BWD_WIDE
-#undef FQ_LAUNCH_BWD
+#define FQ_LAUNCH_BWD_WAVE(NC, REUSE)                                                                       \
+  hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<NC, REUSE>), grid, dim3(256), 0, stream, (const uint16_t*)dy, \
+                     (const uint16_t*)x, (const uint16_t*)gamma, rstd, (uint16_t*)dx, dg_part, M, n, eps)
+#define FQ_BWD_REUSE(LAUNCH, NC) \
+  if (rstd) { LAUNCH(NC, true); } else { LAUNCH(NC, false); }
+  if (n <= 2048) {  // one wave per row, n/512 chunks per lane
+    const int wc = (n / 8 + 63) / 64;
+    if (wc == 1) { FQ_BWD_REUSE(FQ_LAUNCH_BWD_WAVE, 1) }
+    else if (wc == 2) { FQ_BWD_REUSE(FQ_LAUNCH_BWD_WAVE, 2) }
+    else if (wc == 3) { FQ_BWD_REUSE(FQ_LAUNCH_BWD_WAVE, 3) }
+    else { FQ_BWD_REUSE(FQ_LAUNCH_BWD_WAVE, 4) }
+  } else if (n <= 4096) {  // 512 threads per row, one chunk each
+    FQ_BWD_REUSE(FQ_LAUNCH_BWD_BLOCK, 1)
+  } else {  // two chunks each
+    FQ_BWD_REUSE(FQ_LAUNCH_BWD_BLOCK, 2)
+  }
+#undef FQ_BWD_REUSE
+#undef FQ_LAUNCH_BWD_WAVE
+#undef FQ_LAUNCH_BWD_BLOCK
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((n + 63) / 64)), dim3(1024), 0, stream, dg_part, dgamma, (int)P,
