@@ -166,6 +166,18 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
     }
   };
 
+  if constexpr (OUT == 1) {
+    // the quantising form has enough arithmetic per row to want several waves per SIMD:
+    // one row in registers, the other waves cover its loads
+    uint4 buf[NCHUNK];
+    int parity = 0;
+    for (int64_t row = r0; row < r1; row += G) {
+      load_row<T, NCHUNK>(x + row * n, n, buf);
+      process(buf, row, parity);
+      parity ^= 1;
+    }
+    return;
+  }
   uint4 bufA[NCHUNK], bufB[NCHUNK];
   load_row<T, NCHUNK>(x + r0 * n, n, bufA);
   for (int64_t row = r0; row < r1; row += 2 * G) {
@@ -520,6 +532,25 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
     hipLaunchKernelGGL(rowstat_kernel, grid, dim3(64), 0, stream, (const uint16_t*)x, rstd, M, n, eps);
   } else if (!quant) {
     if (reuse_rstd) { FQ_LAUNCH_FWD(true, 0, kE4M3, false) } else { FQ_LAUNCH_FWD(false, 0, kE4M3, false) }
+  } else if (n > 2048) {
+    // wide rows, quantising form: four waves per row (a wave per row needs up to ~230 registers)
+    int64_t wg4 = M;
+    if (wg4 > 256 * 8) wg4 = 256 * 8;
+    const dim3 grid4((unsigned)wg4);
+    const int nc4 = (n / 8 + 255) / 256;
+#define FQ_LAUNCH_FWD4(NC, KINDV, ROUNDV)                                                                      \
+  hipLaunchKernelGGL((rmsnorm_fwd_kernel<256, NC, false, 1, KINDV, ROUNDV>), grid4, dim3(256), 0, stream,       \
+                     (const uint16_t*)x, (const uint16_t*)gamma, out, scale, rstd, M, n, eps, rows_per_wg)
+#define FQ_LAUNCH_FWD4_NC(KINDV, ROUNDV) \
+  if (nc4 == 2) { FQ_LAUNCH_FWD4(2, KINDV, ROUNDV); } else if (nc4 == 3) { FQ_LAUNCH_FWD4(3, KINDV, ROUNDV); } \
+  else { FQ_LAUNCH_FWD4(4, KINDV, ROUNDV); }
+    if (kind == kE5M2) {
+      if (round_scale) { FQ_LAUNCH_FWD4_NC(kE5M2, true) } else { FQ_LAUNCH_FWD4_NC(kE5M2, false) }
+    } else {
+      if (round_scale) { FQ_LAUNCH_FWD4_NC(kE4M3, true) } else { FQ_LAUNCH_FWD4_NC(kE4M3, false) }
+    }
+#undef FQ_LAUNCH_FWD4_NC
+#undef FQ_LAUNCH_FWD4
   } else if (kind == kE5M2) {
     if (round_scale) { FQ_LAUNCH_FWD(false, 1, kE5M2, true) } else { FQ_LAUNCH_FWD(false, 1, kE5M2, false) }
   } else {
