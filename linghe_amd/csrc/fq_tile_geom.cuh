@@ -29,9 +29,8 @@ struct BatchArgs {
 
 // out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
 // backward's dx1|dx2)
-template <bool BATCHED, int THREADS>
-__device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out_w, const BatchArgs& b,
-                                                 ExpertScanShared& scan) {
+template <bool BATCHED>
+__device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out_w, const BatchArgs& b) {
   TileGeom g;
   const int id = blockIdx.x;
   const int rbk = id / ncb;
@@ -49,8 +48,7 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
     g.expert = 0;
     g.valid = left > 0;
   } else {
-    const ExpertTile et = find_expert_tile<THREADS>(b.counts, b.counts_i64, b.n_experts, rbk, scan,
-                                                    b.pad > 1 ? b.pad : 1);
+    const ExpertTile et = find_expert_tile(b.counts, b.counts_i64, b.n_experts, rbk, b.pad > 1 ? b.pad : 1);
     // the lookup's answer is the same in every lane: keep it in scalar registers
     const int expert = uniform32(et.expert), count = uniform32(et.count), rb = uniform32(et.rb);
     const int pcount = uniform32(et.pcount);

@@ -17,8 +17,7 @@ __global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __
                                                               int64_t M, int N, BatchArgs batch) {
   constexpr int RPT = 8;
   __shared__ TileShared<RPT> sh;
-  __shared__ ExpertScanShared scan;
-  const TileGeom g = resolve_tile<BATCHED, 256>(M, N / kGroup, N, batch, scan);
+  const TileGeom g = resolve_tile<BATCHED>(M, N / kGroup, N, batch);
   if (!g.valid) return;
   uint4 raw[RPT];
   load_rows<RPT>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
@@ -43,8 +42,7 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
                                                                 BatchArgs batch) {
   constexpr int RPT = 8;
   __shared__ TileShared<RPT> sh;
-  __shared__ ExpertScanShared scan;
-  const TileGeom g = resolve_tile<true, 256>(M, N / kGroup, N, batch, scan);
+  const TileGeom g = resolve_tile<true>(M, N / kGroup, N, batch);
   if (!g.valid) return;
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
@@ -98,8 +96,7 @@ __global__ __launch_bounds__(512) void silu_quant_fwd_kernel(const uint16_t* __r
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {
   constexpr int RPT = 4;
   __shared__ TileShared<RPT> sh;
-  __shared__ ExpertScanShared scan;
-  const TileGeom g = resolve_tile<BATCHED, 512>(M, n / kGroup, n, batch, scan);
+  const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch);
   if (!g.valid) return;
   const int64_t ld = 2 * (int64_t)n;
   uint4 r1[RPT], r2[RPT];
@@ -147,10 +144,9 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
                                                              int n, BatchArgs batch) {
   constexpr int RPT = 4;
   __shared__ TileShared<RPT> sh;
-  __shared__ ExpertScanShared scan;
   const int nb = n / kGroup;
   const int64_t N = 2 * (int64_t)n;
-  const TileGeom g = resolve_tile<BATCHED, 512>(M, nb, N, batch, scan);
+  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch);
   if (!g.valid) return;
   uint4 r1[RPT], r2[RPT], rgd[RPT];
   const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
@@ -227,9 +223,8 @@ __global__ __launch_bounds__(512) void rmsnorm_quant_tile_kernel(const uint16_t*
                                                                  int64_t M, int n) {
   constexpr int RPT = 4;
   __shared__ TileShared<RPT> sh;
-  __shared__ ExpertScanShared scan;
   BatchArgs none{nullptr, 0, 0};
-  const TileGeom g = resolve_tile<false, 512>(M, n / kGroup, n, none, scan);
+  const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none);
   if (!g.valid) return;
   uint4 raw[RPT];
   load_rows<RPT>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
