@@ -146,7 +146,8 @@ def test_batch_blockwise_quant(gpu, counts):
 
 # ------------------------------------------------------------------ RMSNorm
 @pytest.mark.parametrize("M,N", [(1024, 2048), (1024, 1664), (208, 1664), (512, 4096), (256, 8192),
-                                 (300, 512), (64, 7168), (130, 1536)])
+                                 (300, 512), (64, 7168), (130, 1536), (96, 1024), (40, 128), (3, 2048),
+                                 (70, 3072), (50, 6144)])
 def test_rmsnorm_fwd_bwd(gpu, M, N):
     """reference tests/test_norm.py:114-145 (inputs randn**3, weight randn)."""
     from linghe_amd.utils.norm import triton_rms_norm_backward, triton_rms_norm_forward
@@ -185,7 +186,8 @@ def test_rmsnorm_fwd_bwd(gpu, M, N):
         assert y3.shape == (4, M // 4, N) and torch.equal(y3.view(M, N).cpu(), y.cpu())
 
 
-@pytest.mark.parametrize("M,N", [(1024, 2048), (2048, 1536), (200, 512), (136, 7168), (128, 128)])
+@pytest.mark.parametrize("M,N", [(1024, 2048), (2048, 1536), (200, 512), (136, 7168), (128, 128), (256, 4096),
+                                 (64, 6144), (128, 8192), (72, 2176)])
 @pytest.mark.parametrize("round_scale", [True, False])
 def test_rmsnorm_and_block_quant(gpu, M, N, round_scale):
     """reference tests/test_norm.py:189-220 (x = randn**2, weight randn, modes 0, 1, 2)."""
