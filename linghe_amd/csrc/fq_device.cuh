@@ -23,6 +23,41 @@ template <> struct Fp8Traits<kE5M2Max448> { static constexpr float kMax = 448.0f
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
 
+// Bulk 16-/8-byte accesses with a choice of cache policy.  STREAM adds the
+// non-temporal hint: the line is not kept in L2 or the memory-side cache beyond this
+// access.  For data read once or written once it keeps the caches for what IS reused
+// (the second read of x after a statistic pass, gathered rows, weights); whether it
+// pays is measured per kernel, results are the same either way.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+template <bool STREAM>
+__device__ __forceinline__ uint4 load16(const void* p) {
+  if constexpr (STREAM) {
+    const u32x4_t t = __builtin_nontemporal_load((const u32x4_t*)p);
+    return make_uint4(t.x, t.y, t.z, t.w);
+  } else {
+    return *(const uint4*)p;
+  }
+}
+template <bool STREAM>
+__device__ __forceinline__ void store16(void* p, const uint4& v) {
+  if constexpr (STREAM) {
+    const u32x4_t t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (u32x4_t*)p);
+  } else {
+    *(uint4*)p = v;
+  }
+}
+template <bool STREAM>
+__device__ __forceinline__ void store8(void* p, const uint2& v) {
+  if constexpr (STREAM) {
+    const u32x2_t t = {v.x, v.y};
+    __builtin_nontemporal_store(t, (u32x2_t*)p);
+  } else {
+    *(uint2*)p = v;
+  }
+}
+
 // a value every lane of the workgroup holds identically, moved to scalar registers
 // so that addresses built from it use a scalar base and 32-bit lane offsets
 __device__ __forceinline__ int uniform32(int v) { return __builtin_amdgcn_readfirstlane(v); }

@@ -44,6 +44,14 @@
 
 namespace fq {
 
+// cache policy of the tile loads and of the code stores (see load16/store16)
+#ifndef FQ_NT_STREAM
+#define FQ_NT_STREAM 2
+#endif
+#ifndef FQ_LDNT_STREAM
+#define FQ_LDNT_STREAM 1
+#endif
+
 typedef unsigned long long slot_t;  // low 32 bits: payload, high 32 bits: tag
 
 __device__ __forceinline__ slot_t make_slot(uint32_t v, uint32_t tag) { return (slot_t)v | ((slot_t)tag << 32); }
@@ -108,7 +116,7 @@ __global__ __launch_bounds__(kStreamThreads) void rmsnorm_quant_stream_kernel(
     return t;
   };
   auto issue_loads = [&](const StreamTile& t, uint4 (&raw)[RPT]) {
-    load_rows<RPT>(x + t.row0 * n + (int64_t)t.cb * kGroup, n, t.rows_valid, raw);
+    load_rows<RPT, FQ_LDNT_STREAM != 0>(x + t.row0 * n + (int64_t)t.cb * kGroup, n, t.rows_valid, raw);
   };
   // stage A: partial sums of the tile's rows -> part[slab][row][cb]
   auto publish_partials = [&](const StreamTile& t, const uint4 (&raw)[RPT]) {
@@ -241,7 +249,7 @@ __global__ __launch_bounds__(kStreamThreads) void rmsnorm_quant_stream_kernel(
     g.st_row = t.slab;
     g.expert = 0;
     g.valid = true;
-    quantize_tile<KIND, ROUND, 2, RPT>(v, make_out(out, g, n, t.cb), sh);
+    quantize_tile<KIND, ROUND, 2, RPT, FQ_NT_STREAM>(v, make_out(out, g, n, t.cb), sh);
   };
 
   // three tiles in registers with fixed roles: ra = tile i+1 (arriving), rw = tile i

@@ -33,6 +33,15 @@
 
 namespace fq {
 
+// cache policy (see load16/store16): FQ_ROUTER_NT puts the non-temporal hint on the
+// stores of y and the codes, FQ_ROUTER_LDNT on the loads of x in the resident kernel
+#ifndef FQ_ROUTER_NT
+#define FQ_ROUTER_NT 1
+#endif
+#ifndef FQ_ROUTER_LDNT
+#define FQ_ROUTER_LDNT 1
+#endif
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx16_t __attribute__((ext_vector_type(16)));
 
@@ -189,11 +198,11 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
       const int slot = ahalf * 32 + ((RPT * rg + u) ^ aj);
       sh.a[buf][0][aj][slot] = hi;
       sh.a[buf][1][aj][slot] = pack8_bf16(lo);
-      *(uint4*)(yrow + (int64_t)u * K + kb * kGroup) = hi;
+      store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, hi);
       uint2 pk;
       pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
       pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
-      *(uint2*)(qrow + (int64_t)u * K + kb * kGroup) = pk;
+      store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
       if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
     }
     __syncthreads();
@@ -295,7 +304,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
   auto w_piece = [&](int kb, int t, int j) { return wlane[((int64_t)kb * WAVES * NT + t) * 8 * 64 + j * 64]; };
   auto fetch_x = [&](int kb, uint4 (&xk)[RPT]) {
 #pragma unroll
-    for (int u = 0; u < RPT; ++u) xk[u] = *(const uint4*)(xrow + (int64_t)u * K + kb * kGroup);
+    for (int u = 0; u < RPT; ++u) xk[u] = load16<FQ_ROUTER_LDNT != 0>(xrow + (int64_t)u * K + kb * kGroup);
   };
 #pragma unroll
   for (int d = 0; d < kWAhead; ++d)
@@ -408,11 +417,11 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
         const Divisor d = make_divisor(sc);
 #pragma unroll
         for (int i = 0; i < 8; ++i) qv[i] = div_by_scale<ROUND>(yv[i], d);
-        *(uint4*)(yrow + (int64_t)u * K + kb * kGroup) = pack8_bf16(yv);
+        store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, pack8_bf16(yv));
         uint2 pk;
         pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
         pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
-        *(uint2*)(qrow + (int64_t)u * K + kb * kGroup) = pk;
+        store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
         if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
       }
     }

@@ -66,7 +66,17 @@ struct __attribute__((packed, aligned(1))) Bytes16 { uint32_t x, y, z, w; };
 struct __attribute__((packed, aligned(1))) Bytes8 { uint32_t x, y; };
 struct __attribute__((packed, aligned(1))) Bytes4 { uint32_t x; };
 struct __attribute__((packed, aligned(1))) Bytes2 { uint16_t x; };
-__device__ __forceinline__ void store16_any(uint8_t* dst, const uint4& v) { *(Bytes16*)dst = Bytes16{v.x, v.y, v.z, v.w}; }
+// STREAM: with the non-temporal hint (fq_device.cuh)
+typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(1)));
+template <bool STREAM>
+__device__ __forceinline__ void store16_any(uint8_t* dst, const uint4& v) {
+  if constexpr (STREAM) {
+    const u32x4_any t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (u32x4_any*)dst);
+  } else {
+    *(Bytes16*)dst = Bytes16{v.x, v.y, v.z, v.w};
+  }
+}
 
 // dword k (k = 0..3, lane-variable) of a 16-byte chunk held in four registers
 __device__ __forceinline__ uint32_t pick_dword(const uint4& v, int k) {
@@ -80,13 +90,14 @@ __device__ __forceinline__ uint32_t pick_dword(const uint4& v, int k) {
 // Called by the 8 threads ch = 0..7 that share the row: thread ch owns source
 // bytes [16 ch, 16 ch + 16); a chunk cut by the end of the row leaves as at most
 // one 8-, 4-, 2- and 1-byte store.
+template <bool STREAM>
 __device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uint8_t* dst_row, int len, int ch) {
   const int rem = len - 16 * ch;
   if (rem <= 0) return;
   const uint4 v = *(const uint4*)(lds_row + ((ch ^ swz) * 16));
   uint8_t* dst = dst_row + 16 * ch;
   if (rem >= 16) {
-    store16_any(dst, v);
+    store16_any<STREAM>(dst, v);
     return;
   }
   int p = 0;
@@ -99,7 +110,7 @@ __device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uin
 // Quantise the tile held in registers (v[s][j] = element (rg*RPT+s, cg*8+j);
 // rows >= rows_valid must hold 0).  All threads of the workgroup must call it.
 // FULL: the tile has all 128 rows, so no load or store needs a mask.
-template <int KIND, bool ROUND, int MODE, int RPT, bool FULL>
+template <int KIND, bool ROUND, int MODE, int RPT, bool FULL, int NT>
 __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], const TileOut& o,
                                                    TileShared<RPT>& sh) {
   using Shape = TileShape<RPT>;
@@ -154,7 +165,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
       const int i = rg * RPT + s;
       // scalar tile base + 32-bit lane offset (128 rows of at most 2^23 bytes)
-      if (FULL || i < o.rows_valid) *(uint2*)((o.q + o.q_off) + ((uint32_t)i * (uint32_t)o.q_ld + (uint32_t)cg * 8u)) = pk;
+      if (FULL || i < o.rows_valid) store8<(NT & 2) != 0>((o.q + o.q_off) + ((uint32_t)i * (uint32_t)o.q_ld + (uint32_t)cg * 8u), pk);
     }
   }
 
@@ -230,22 +241,23 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       if constexpr (FULL) {
         const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
         // scalar tile base + 32-bit lane offset (128 transposed rows of at most 2^24 bytes)
-        store16_any((o.qt + o.t_off) + ((uint32_t)c * (uint32_t)o.t_ld + (uint32_t)ch * 16u), val);
+        store16_any<(NT & 1) != 0>((o.qt + o.t_off) + ((uint32_t)c * (uint32_t)o.t_ld + (uint32_t)ch * 16u), val);
       } else {
-        store_t_row(sh.t + c * kGroup, (c >> 3) & 7, (o.qt + o.t_off) + (uint32_t)c * (uint32_t)o.t_ld, o.rows_valid, ch);
+        store_t_row<(NT & 1) != 0>(sh.t + c * kGroup, (c >> 3) & 7, (o.qt + o.t_off) + (uint32_t)c * (uint32_t)o.t_ld, o.rows_valid, ch);
       }
     }
     __syncthreads();  // LDS is reused by a following call
   }
 }
 
-template <int KIND, bool ROUND, int MODE, int RPT>
+// NT: bit 0 = transposed codes, bit 1 = row-wise codes leave with the non-temporal hint
+template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0>
 __device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o,
                                               TileShared<RPT>& sh) {
   // workgroup-uniform choice of the mask-free path
   const bool full = o.rows_valid == kGroup;
-  if (full) quantize_tile_impl<KIND, ROUND, MODE, RPT, true>(v, o, sh);
-  else quantize_tile_impl<KIND, ROUND, MODE, RPT, false>(v, o, sh);
+  if (full) quantize_tile_impl<KIND, ROUND, MODE, RPT, true, NT>(v, o, sh);
+  else quantize_tile_impl<KIND, ROUND, MODE, RPT, false, NT>(v, o, sh);
 }
 
 // ---------------------------------------------------------------------------

@@ -95,7 +95,8 @@ __device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g,
 }
 
 // RPT rows x 8 bf16 columns of a row-major matrix; rows >= rows_valid read as 0
-template <int RPT>
+// STREAM: loads carry the non-temporal hint (the tile is not read again)
+template <int RPT, bool STREAM = false>
 __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
@@ -107,12 +108,12 @@ __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int 
   const uint32_t off0 = (uint32_t)(rg * RPT) * pitch + (uint32_t)cg * 16u;
   if (rows_valid == kGroup) {  // workgroup-uniform: no per-row masks
 #pragma unroll
-    for (int s = 0; s < RPT; ++s) raw[s] = *(const uint4*)(b + (off0 + (uint32_t)s * pitch));
+    for (int s = 0; s < RPT; ++s) raw[s] = load16<STREAM>(b + (off0 + (uint32_t)s * pitch));
   } else {
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
       raw[s] = make_uint4(0, 0, 0, 0);
-      if (rg * RPT + s < rows_valid) raw[s] = *(const uint4*)(b + (off0 + (uint32_t)s * pitch));
+      if (rg * RPT + s < rows_valid) raw[s] = load16<STREAM>(b + (off0 + (uint32_t)s * pitch));
     }
   }
 }

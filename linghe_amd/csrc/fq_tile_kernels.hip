@@ -7,6 +7,45 @@
 #include "fq_tile_geom.cuh"
 #include "fq_launch.h"
 
+// Cache policy per kernel, chosen by measurement (cold inputs, MI355X).
+//   FQ_NT_<kernel>: which code stores carry the non-temporal hint (bit 0: transposed
+//   codes, bit 1: row-wise codes).  With it the outputs do not displace inputs from L2
+//   and the memory-side cache: gather+pad+quant 75 -> 55 us, RMSNorm+quant after the
+//   statistic pass 25 -> 21 us (8192 x 2048) and 146 -> 122 us (16384 x 7168).  The
+//   SwiGLU backward is 3-7 % slower when its transposed stores carry it, the plain
+//   blockwise quantisers 10-17 % slower with any of it.
+//   FQ_LDNT_<kernel>: the bulk loads carry it (3-5 % on the SwiGLU kernels and the
+//   RMSNorm tile kernel, nothing on the plain quantisers).
+#ifndef FQ_NT_BLOCKWISE
+#define FQ_NT_BLOCKWISE 0
+#endif
+#ifndef FQ_NT_PERMUTE
+#define FQ_NT_PERMUTE 3
+#endif
+#ifndef FQ_NT_SILU_FWD
+#define FQ_NT_SILU_FWD 3
+#endif
+#ifndef FQ_NT_SILU_BWD
+#define FQ_NT_SILU_BWD 2
+#endif
+#ifndef FQ_NT_RMSNORM
+#define FQ_NT_RMSNORM 3
+#endif
+#ifndef FQ_LDNT_BLOCKWISE
+#define FQ_LDNT_BLOCKWISE 0
+#endif
+#ifndef FQ_LDNT_PERMUTE
+#define FQ_LDNT_PERMUTE 0
+#endif
+#ifndef FQ_LDNT_SILU_FWD
+#define FQ_LDNT_SILU_FWD 1
+#endif
+#ifndef FQ_LDNT_SILU_BWD
+#define FQ_LDNT_SILU_BWD 1
+#endif
+#ifndef FQ_LDNT_RMSNORM
+#define FQ_LDNT_RMSNORM 1
+#endif
 namespace fq {
 
 // ---------------------------------------------------------------------------
@@ -20,11 +59,11 @@ __global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __
   const TileGeom g = resolve_tile<BATCHED>(M, N / kGroup, N, batch);
   if (!g.valid) return;
   uint4 raw[RPT];
-  load_rows<RPT>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
+  load_rows<RPT, FQ_LDNT_BLOCKWISE != 0>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
-  quantize_tile<KIND, ROUND, MODE, RPT>(v, make_out(out, g, N, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_BLOCKWISE>(v, make_out(out, g, N, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -63,7 +102,7 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
     raw[s] = make_uint4(0, 0, 0, 0);
     // rows of the padding, and indices that do not name a source row, read as zero
     if (rg * RPT + s < g.rows_valid && (uint32_t)src[s] < (uint64_t)src_rows)
-      raw[s] = *(const uint4*)(col + (int64_t)src[s] * N);
+      raw[s] = load16<FQ_LDNT_PERMUTE != 0>(col + (int64_t)src[s] * N);
   }
   if (probs != nullptr && g.cb == 0 && threadIdx.x < kGroup) {
     const int i = threadIdx.x;
@@ -85,7 +124,7 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
-  quantize_tile<KIND, ROUND, 2, RPT>(v, make_out(out, g, N, g.cb), sh);
+  quantize_tile<KIND, ROUND, 2, RPT, FQ_NT_PERMUTE>(v, make_out(out, g, N, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -101,8 +140,8 @@ __global__ __launch_bounds__(512) void silu_quant_fwd_kernel(const uint16_t* __r
   const int64_t ld = 2 * (int64_t)n;
   uint4 r1[RPT], r2[RPT];
   const uint16_t* p = x + g.row0 * ld + (int64_t)g.cb * kGroup;
-  load_rows<RPT>(p, ld, g.rows_valid, r1);
-  load_rows<RPT>(p + n, ld, g.rows_valid, r2);
+  load_rows<RPT, FQ_LDNT_SILU_FWD != 0>(p, ld, g.rows_valid, r1);
+  load_rows<RPT, FQ_LDNT_SILU_FWD != 0>(p + n, ld, g.rows_valid, r2);
   const int rg = threadIdx.x >> 4;
   float v[RPT][8];
 #pragma unroll
@@ -128,7 +167,7 @@ __global__ __launch_bounds__(512) void silu_quant_fwd_kernel(const uint16_t* __r
       }
     }
   }
-  quantize_tile<KIND, ROUND, MODE, RPT>(v, make_out(out, g, n, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_SILU_FWD>(v, make_out(out, g, n, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -150,9 +189,9 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   if (!g.valid) return;
   uint4 r1[RPT], r2[RPT], rgd[RPT];
   const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
-  load_rows<RPT>(p, N, g.rows_valid, r1);
-  load_rows<RPT>(p + n, N, g.rows_valid, r2);
-  load_rows<RPT>(gr + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, rgd);
+  load_rows<RPT, FQ_LDNT_SILU_BWD != 0>(p, N, g.rows_valid, r1);
+  load_rows<RPT, FQ_LDNT_SILU_BWD != 0>(p + n, N, g.rows_valid, r2);
+  load_rows<RPT, FQ_LDNT_SILU_BWD != 0>(gr + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, rgd);
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
   float d1[RPT][8], d2[RPT][8];
@@ -197,8 +236,8 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
       if (i < g.rows_valid) dw_part[(g.row0 + i) * nb + g.cb] = my_dw;
     }
   }
-  quantize_tile<KIND, ROUND, 2, RPT>(d1, make_out(out, g, N, g.cb), sh);
-  quantize_tile<KIND, ROUND, 2, RPT>(d2, make_out(out, g, N, nb + g.cb), sh);
+  quantize_tile<KIND, ROUND, 2, RPT, FQ_NT_SILU_BWD>(d1, make_out(out, g, N, g.cb), sh);
+  quantize_tile<KIND, ROUND, 2, RPT, FQ_NT_SILU_BWD>(d2, make_out(out, g, N, nb + g.cb), sh);
 }
 
 // dw[r] = sum_b part[r, b]  (fixed order), stored as fp32 or bf16
@@ -227,7 +266,7 @@ __global__ __launch_bounds__(512) void rmsnorm_quant_tile_kernel(const uint16_t*
   const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none);
   if (!g.valid) return;
   uint4 raw[RPT];
-  load_rows<RPT>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
+  load_rows<RPT, FQ_LDNT_RMSNORM != 0>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
   float gm[8];
@@ -242,7 +281,7 @@ __global__ __launch_bounds__(512) void rmsnorm_quant_tile_kernel(const uint16_t*
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[s][j] = (a[j] * r) * gm[j];
   }
-  quantize_tile<KIND, ROUND, MODE, RPT>(v, make_out(out, g, n, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_RMSNORM>(v, make_out(out, g, n, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
