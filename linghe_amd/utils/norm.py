@@ -18,7 +18,7 @@ _MAX_HIDDEN = 8192  # the reference asserts next_power_of_2(n) <= 8192
 #          variant on MI355X at every size tried;
 #   True   hand the library its workspace, so that the call is ONE pass over x (the
 #          statistic is exchanged between workgroups inside the kernel):
-#          algorithmic HBM traffic, 20-25 % slower at the sizes measured.
+#          algorithmic HBM traffic, 45-60 % slower at the sizes measured.
 SINGLE_PASS = False
 
 
