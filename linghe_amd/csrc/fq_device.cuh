@@ -28,35 +28,35 @@ __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(
 // access.  For data read once or written once it keeps the caches for what IS reused
 // (the second read of x after a statistic pass, gathered rows, weights); whether it
 // pays is measured per kernel, results are the same either way.
+// Every pointer these helpers see is device memory: the explicit global address
+// space keeps the accesses global_load/global_store when the pointer was rebuilt from
+// scalar registers (a generic pointer would make them flat accesses).
+#define FQ_GLOBAL __attribute__((address_space(1)))
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 template <bool STREAM>
 __device__ __forceinline__ uint4 load16(const void* p) {
-  if constexpr (STREAM) {
-    const u32x4_t t = __builtin_nontemporal_load((const u32x4_t*)p);
-    return make_uint4(t.x, t.y, t.z, t.w);
-  } else {
-    return *(const uint4*)p;
-  }
+  const FQ_GLOBAL u32x4_t* g = (const FQ_GLOBAL u32x4_t*)p;
+  u32x4_t t;
+  if constexpr (STREAM) t = __builtin_nontemporal_load(g);
+  else t = *g;
+  return make_uint4(t.x, t.y, t.z, t.w);
 }
 template <bool STREAM>
 __device__ __forceinline__ void store16(void* p, const uint4& v) {
-  if constexpr (STREAM) {
-    const u32x4_t t = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(t, (u32x4_t*)p);
-  } else {
-    *(uint4*)p = v;
-  }
+  FQ_GLOBAL u32x4_t* g = (FQ_GLOBAL u32x4_t*)p;
+  const u32x4_t t = {v.x, v.y, v.z, v.w};
+  if constexpr (STREAM) __builtin_nontemporal_store(t, g);
+  else *g = t;
 }
 template <bool STREAM>
 __device__ __forceinline__ void store8(void* p, const uint2& v) {
-  if constexpr (STREAM) {
-    const u32x2_t t = {v.x, v.y};
-    __builtin_nontemporal_store(t, (u32x2_t*)p);
-  } else {
-    *(uint2*)p = v;
-  }
+  FQ_GLOBAL u32x2_t* g = (FQ_GLOBAL u32x2_t*)p;
+  const u32x2_t t = {v.x, v.y};
+  if constexpr (STREAM) __builtin_nontemporal_store(t, g);
+  else *g = t;
 }
+__device__ __forceinline__ void store_f32(float* p, float v) { *(FQ_GLOBAL float*)p = v; }
 
 // a value every lane of the workgroup holds identically, moved to scalar registers
 // so that addresses built from it use a scalar base and 32-bit lane offsets
@@ -119,7 +119,9 @@ __device__ __forceinline__ float sumsq8(const uint4& p) {
 // 4 fp32 -> 4 fp8 codes in one dword (native converts, RNE)
 template <int KIND>
 __device__ __forceinline__ uint32_t pack4_fp8(float a, float b, float c, float d) {
-  uint32_t w = 0;
+  // both halves of w are written by the two converts; seeding it with a's bits (a is
+  // dead after this) lets the first convert work in place instead of clearing a register
+  uint32_t w = as_u32(a);
   if constexpr (!Fp8Traits<KIND>::kBf8) {
     w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
     w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);

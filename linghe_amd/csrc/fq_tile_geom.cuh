@@ -95,16 +95,20 @@ __device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g,
 }
 
 // RPT rows x 8 bf16 columns of a row-major matrix; rows >= rows_valid read as 0
-// STREAM: loads carry the non-temporal hint (the tile is not read again)
-template <int RPT, bool STREAM = false>
+// STREAM: loads carry the non-temporal hint (the tile is not read again).
+// SCALAR: the tile base, the same in every lane, is moved to scalar registers
+template <int RPT, bool STREAM = false, bool SCALAR = true>
 __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
-  // base is the same for the whole workgroup (scalar registers); a tile spans at
-  // most 128 rows of at most 2^24 bytes (the widest input the entry points accept),
-  // so lane offsets fit 32 bits
+  // a tile spans at most 128 rows of at most 2^24 bytes (the widest input the entry
+  // points accept), so lane offsets fit 32 bits
   const uint8_t* b = (const uint8_t*)base;
-  const uint32_t pitch = (uint32_t)ld * 2u;
+  uint32_t pitch = (uint32_t)ld * 2u;
+  if constexpr (SCALAR) {
+    b = (const uint8_t*)uniform64((int64_t)b);
+    pitch = (uint32_t)uniform32((int)pitch);
+  }
   const uint32_t off0 = (uint32_t)(rg * RPT) * pitch + (uint32_t)cg * 16u;
   if (rows_valid == kGroup) {  // workgroup-uniform: no per-row masks
 #pragma unroll

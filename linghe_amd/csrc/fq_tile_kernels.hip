@@ -31,6 +31,13 @@
 #ifndef FQ_NT_RMSNORM
 #define FQ_NT_RMSNORM 3
 #endif
+//   FQ_LEAN_BLOCKWISE: the lean form of the quantiser and of the tile loads (scalar
+//   bases, paired column-maximum reduction; every other tile kernel uses it, -3 to -9 %)
+//   in the PLAIN blockwise quantiser, which is 7 % slower with it (48 -> 51 us at
+//   65536 x 1024); the per-expert form takes it (zipf counts: 60.6 -> 57.9 us).
+#ifndef FQ_LEAN_BLOCKWISE
+#define FQ_LEAN_BLOCKWISE 0
+#endif
 #ifndef FQ_LDNT_BLOCKWISE
 #define FQ_LDNT_BLOCKWISE 0
 #endif
@@ -59,11 +66,11 @@ __global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __
   const TileGeom g = resolve_tile<BATCHED>(M, N / kGroup, N, batch);
   if (!g.valid) return;
   uint4 raw[RPT];
-  load_rows<RPT, FQ_LDNT_BLOCKWISE != 0>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
+  load_rows<RPT, FQ_LDNT_BLOCKWISE != 0, BATCHED || FQ_LEAN_BLOCKWISE != 0>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
-  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_BLOCKWISE>(v, make_out(out, g, N, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_BLOCKWISE, BATCHED || FQ_LEAN_BLOCKWISE != 0>(v, make_out(out, g, N, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
