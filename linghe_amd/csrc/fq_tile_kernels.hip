@@ -53,6 +53,17 @@
 #ifndef FQ_LDNT_RMSNORM
 #define FQ_LDNT_RMSNORM 1
 #endif
+// Rows per thread (workgroup = 2048 / RPT threads).  With the outputs streamed past
+// the caches the tile kernels are bound by vector-instruction issue, and 8 rows per
+// thread spread the per-thread overhead over twice the elements: the RMSNorm tile
+// kernel (93 registers, five 256-thread workgroups per CU) gains 3-4 %; the SwiGLU
+// forward needs 135 registers in that shape and loses 5 %.
+#ifndef FQ_RPT_FWD
+#define FQ_RPT_FWD 4
+#endif
+#ifndef FQ_RPT_RMS
+#define FQ_RPT_RMS 8
+#endif
 namespace fq {
 
 // ---------------------------------------------------------------------------
@@ -138,9 +149,9 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
 // SwiGLU forward + quant.  y = (sigmoid(x1)*x1)*x2 [*w_row]   (fp32)
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED>
-__global__ __launch_bounds__(512) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
+__global__ __launch_bounds__(2048 / FQ_RPT_FWD) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {
-  constexpr int RPT = 4;
+  constexpr int RPT = FQ_RPT_FWD;
   __shared__ TileShared<RPT> sh;
   const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch);
   if (!g.valid) return;
@@ -263,11 +274,11 @@ __global__ __launch_bounds__(256) void rowsum_kernel(const float* __restrict__ p
 //   y = (x * rstd[row]) * gamma[col]
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, int MODE>
-__global__ __launch_bounds__(512) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
+__global__ __launch_bounds__(2048 / FQ_RPT_RMS) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
                                                                  const uint16_t* __restrict__ gamma,
                                                                  const float* __restrict__ rstd, OutPtrs out,
                                                                  int64_t M, int n) {
-  constexpr int RPT = 4;
+  constexpr int RPT = FQ_RPT_RMS;
   __shared__ TileShared<RPT> sh;
   BatchArgs none{nullptr, 0, 0};
   const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none);
@@ -337,7 +348,7 @@ hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_b
   RowWeight w{weight, weight_bf16};
   const int64_t tiles = row_blocks * (n / kGroup);
   if (tiles == 0) return hipSuccess;
-  const dim3 grid((unsigned)tiles), block(512);
+  const dim3 grid((unsigned)tiles), block(2048 / FQ_RPT_FWD);
   const bool batched = counts != nullptr;
   const bool weighted = weight != nullptr;
   FQ_DISPATCH_KIND(kind, K,
@@ -383,7 +394,7 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
   const int64_t tiles = ((M + kGroup - 1) / kGroup) * (n / kGroup);
   if (tiles == 0) return hipSuccess;
-  const dim3 grid((unsigned)tiles), block(512);
+  const dim3 grid((unsigned)tiles), block(2048 / FQ_RPT_RMS);
   FQ_DISPATCH_KIND(kind, K,
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
