@@ -26,7 +26,7 @@ def triton_block_quant(x, block_size=128, round_scale=False, *, fp8_dtype=torch.
     _lib.require_device_bf16(x, "x")
     y = torch.empty((M, N), dtype=fp8_dtype, device=x.device)
     s = torch.empty(M // block_size, N // block_size, dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.lib.fq_block_quant(_lib.ptr(x), _lib.ptr(y), _lib.ptr(s), M, N, int(bool(round_scale)),
                                            _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
     return y, s
@@ -57,7 +57,7 @@ def triton_blockwise_quant(x, round_scale=False, output_mode=2, *, fp8_dtype=tor
     xt_q = torch.empty((N, M), device=device, dtype=fp8_dtype)
     xt_scale = torch.empty(((M + 127) // 128, N), device=device, dtype=torch.float32)
     if M > 0:
-        with torch.cuda.device(device):
+        with _lib.on_device(device):
             _lib.check(_lib.lib.fq_blockwise_quant(
                 _lib.ptr(x), _lib.ptr(x_q), _lib.ptr(x_scale), _lib.ptr(xt_q), _lib.ptr(xt_scale), M, N,
                 int(bool(round_scale)), output_mode, _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
@@ -97,7 +97,7 @@ def triton_batch_blockwise_quant(xs, token_count_per_expert, splits, round_scale
         is64 = 0
     else:
         raise TypeError(f"token_count_per_expert must be int32 or int64, got {counts.dtype}")
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         _lib.check(_lib.lib.fq_batched_blockwise_quant(
             _lib.ptr(xs), _lib.ptr(counts), is64, n_experts, blocks, _lib.ptr(x_q), _lib.ptr(x_scale),
             _lib.ptr(xt_q), _lib.ptr(xt_scale), M, N, int(bool(round_scale)), _lib.fp8_kind(fp8_dtype),

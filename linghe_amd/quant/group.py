@@ -29,7 +29,7 @@ def triton_group_quant(x, dtype=torch.float8_e4m3fn, group_size=128, round_scale
     y = torch.empty((M, N), device=x.device, dtype=dtype)
     s = torch.empty(M, N // group_size, device=x.device, dtype=torch.float32)
     if M > 0:
-        with torch.cuda.device(x.device):
+        with _lib.on_device(x.device):
             _lib.check(_lib.lib.fq_group_quant(_lib.ptr(x), _lib.ptr(y), _lib.ptr(s), M, N,
                                                int(bool(round_scale)),
                                                _lib.FQ_E4M3 if dtype == torch.float8_e4m3fn else _lib.FQ_E5M2_MAX448,

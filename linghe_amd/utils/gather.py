@@ -66,7 +66,7 @@ def triton_batch_block_pad_permute_with_indices(
             pbf16 = 1
         elif probs.dtype != torch.float32:
             raise TypeError(f"probs must be float32 or bfloat16, got {probs.dtype}")
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         _lib.check(_lib.lib.fq_batched_pad_permute_quant(
             _lib.ptr(xs), _lib.ptr(counts), is64, n_experts, blocks, _lib.ptr(indices),
             _lib.ptr(probs), pbf16, _lib.ptr(prob_output), _lib.ptr(x_q), _lib.ptr(x_scale), _lib.ptr(xt_q),

@@ -59,7 +59,7 @@ def triton_rms_norm_forward(x, weight, eps=1e-6, out=None, rms=None):
     if not reuse:
         rms = torch.empty((M,), device=x.device, dtype=torch.float32)
     if M > 0:
-        with torch.cuda.device(x.device):
+        with _lib.on_device(x.device):
             _lib.check(_lib.lib.fq_rmsnorm_fwd(_lib.ptr(x), _lib.ptr(weight), _lib.ptr(out), _lib.ptr(rms),
                                                M, n, float(eps), int(reuse), _lib.stream_of(x)))
     return out, rms
@@ -83,7 +83,7 @@ def triton_rms_norm_backward(grad_output, x, w, eps=1e-6, rms=None):
     dw = torch.empty((n,), dtype=torch.float32, device=w.device)
     n_part = int(_lib.lib.fq_rmsnorm_bwd_num_partials(M, n))
     tmp_dw = torch.empty((n_part, n), dtype=torch.float32, device=w.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.lib.fq_rmsnorm_bwd(_lib.ptr(grad_output), _lib.ptr(x), _lib.ptr(w), _lib.ptr(rms),
                                            _lib.ptr(dx), _lib.ptr(dw), _lib.ptr(tmp_dw), n_part, M, n,
                                            float(eps), _lib.stream_of(x)))
@@ -152,7 +152,7 @@ def triton_rms_norm_and_block_quant_forward(
         rms = torch.empty((M,), dtype=torch.float32, device=device)
 
     if M > 0:
-        with torch.cuda.device(device):
+        with _lib.on_device(device):
             ws, ws_bytes = (None, 0)
             if output_mode == 2 and SINGLE_PASS:
                 ws, ws_bytes = _lib.norm_workspace(x, M, n)
@@ -218,7 +218,7 @@ def triton_rms_norm_fp32_gemm_block_quant_forward(
     xt_s = torch.empty((M // 128, K), device=device, dtype=torch.float32)
     if M == 0:
         return y, rms, logits, x_q, x_s, xt_q, xt_s
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         if output_mode == 0:
             _lib.require_device_bf16(route_weight, "route_weight")
             assert N <= 512, f"{N=} router outputs: at most 512 are supported"

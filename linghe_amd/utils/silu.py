@@ -50,7 +50,7 @@ def triton_weighted_silu_forward(x, weight=None, out=None, asm=False):
     if weight is not None:
         assert weight.is_contiguous() and weight.numel() == M
         wflag = _weight_flag(weight)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.lib.fq_swiglu_fwd(_lib.ptr(x), _lib.ptr(weight), wflag, _lib.ptr(out), M, N // 2,
                                           _lib.stream_of(x)))
     return out
@@ -80,7 +80,7 @@ def triton_weighted_silu_backward(g, x, weight=None):
         wflag = _weight_flag(weight)
         dw = torch.empty(weight.shape, device=x.device, dtype=weight.dtype)
     dx = torch.empty((M, N), device=x.device, dtype=x.dtype)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.lib.fq_swiglu_bwd(_lib.ptr(g), _lib.ptr(x), _lib.ptr(weight), wflag, _lib.ptr(dx),
                                           _lib.ptr(dw), M, N // 2, _lib.stream_of(x)))
     return dx, dw
@@ -119,7 +119,7 @@ def triton_silu_and_block_quant_forward(
     transpose_output = torch.empty((n, M), device=device, dtype=fp8_dtype)
     transpose_scale = torch.empty(((M + 127) // 128, n), device=device, dtype=torch.float32)
     if M > 0:
-        with torch.cuda.device(device):
+        with _lib.on_device(device):
             _lib.check(_lib.lib.fq_swiglu_quant_fwd(
                 _lib.ptr(x), _lib.ptr(out), _lib.ptr(scale), _lib.ptr(transpose_output),
                 _lib.ptr(transpose_scale), M, n, int(bool(round_scale)), output_mode,
@@ -155,7 +155,7 @@ def triton_silu_and_block_quant_backward(g, x, round_scale=False, *, fp8_dtype=t
     transpose_dx = torch.empty((N, M), device=device, dtype=fp8_dtype)
     transpose_dx_scale = torch.empty(((M + 127) // 128, N), device=device, dtype=torch.float32)
     if M > 0:
-        with torch.cuda.device(device):
+        with _lib.on_device(device):
             _lib.check(_lib.lib.fq_swiglu_quant_bwd(
                 _lib.ptr(g), _lib.ptr(x), _lib.ptr(dx), _lib.ptr(dx_scale), _lib.ptr(transpose_dx),
                 _lib.ptr(transpose_dx_scale), M, n, int(bool(round_scale)), _lib.fp8_kind(fp8_dtype),
@@ -211,7 +211,7 @@ def triton_batch_weighted_silu_and_block_quant_forward(
     transpose_scale = torch.empty((blocks, n), device=device, dtype=torch.float32)
     if M == 0:
         return out, scale, transpose_output, transpose_scale
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         _lib.check(_lib.lib.fq_batched_swiglu_quant_fwd(
             _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(counts), _counts_flag(counts),
             n_experts, blocks, _lib.ptr(out), _lib.ptr(scale), _lib.ptr(transpose_output),
@@ -251,7 +251,7 @@ def triton_batch_weighted_silu_and_block_quant_backward(
     if s == 0:
         return dx, dx_scale, dw, transpose_dx, transpose_dx_scale
     dws = torch.empty((M, n // 128), device=device, dtype=torch.float32)
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         _lib.check(_lib.lib.fq_batched_swiglu_quant_bwd(
             _lib.ptr(g), _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(counts),
             _counts_flag(counts), n_expert, s, _lib.ptr(dx), _lib.ptr(dx_scale), _lib.ptr(dw),
