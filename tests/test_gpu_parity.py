@@ -125,7 +125,9 @@ def test_group_quant(gpu, M, N, round_scale):
 
 
 @pytest.mark.parametrize("counts", [[128, 0, 256, 16, 0, 144, 1, 127], [0, 0, 0, 0], [300],
-                                    [33, 65, 7, 129, 513, 2, 0, 90, 128, 128, 77, 5, 0, 0, 250, 31]])
+                                    [33, 65, 7, 129, 513, 2, 0, 90, 128, 128, 77, 5, 0, 0, 250, 31],
+                                    # every length of a ragged transposed row modulo 16, alone and after a full block
+                                    list(range(1, 17)) + [128 + r for r in range(1, 16)] + [113, 120, 126]])
 def test_batch_blockwise_quant(gpu, counts):
     from linghe_amd.quant.block import triton_batch_blockwise_quant
 
@@ -414,6 +416,7 @@ def _batched_case(gpu, counts, N, coef, gcoef, seed, wdtype=torch.float32):
     ([144, 80, 400, 16], 1536, 100.0, 100.0),
     ([144, 80, 400, 16], 1536, 0.0, 0.0),
     ([37, 0, 129, 1, 255, 3], 512, 1.0, 1e-3),   # counts that are not multiples of 16
+    (list(range(1, 17)) + [128 + r for r in (1, 2, 3, 6, 9, 12, 15)], 256, 1.0, 1.0),   # every ragged tail
     ([64, 64], 8192, 1.0, 1.0),
 ])
 def test_batch_weighted_silu_and_block_quant(gpu, counts, N, coef, gcoef):
