@@ -344,7 +344,7 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
 // Which expert owns the global 128-row block `blk` (blocks are numbered expert
 // after expert, ceil(count/128) per expert)?  Computed from the device-side
 // counts by a prefix scan that EVERY WAVE runs for itself, 64 experts per step with
-// the loads of four steps in flight together: no LDS, no barrier, and every
+// the loads of up to sixteen steps in flight together: no LDS, no barrier, and every
 // thread of the workgroup ends with the same answer.  (A workgroup-wide scan
 // with three barriers cost 13 % of the batched SwiGLU forward.)  An out-of-range
 // blk (host and device counts disagree) yields expert = -1.
@@ -362,19 +362,27 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
   t.row_start = 0;
   t.tblock_start = 0;
   int run_rows = 0, run_blocks = 0;
-  for (int base0 = 0; base0 < n_experts; base0 += 256) {
-    int c4[4];
+  // the counts of up to 1024 experts (16 steps) are fetched together: one memory round
+  // trip however many steps the scan then takes
+  constexpr int kSteps = 16;
+  for (int base0 = 0; base0 < n_experts; base0 += 64 * kSteps) {
+    const int left = n_experts - base0;
+    const int steps = left >= 64 * kSteps ? kSteps : (left + 63) / 64;  // wave-uniform
+    int cs[kSteps];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int e = base0 + k * 64 + lane;
-      c4[k] = (e < n_experts) ? load_count(counts, is_i64, e) : 0;
+    for (int k = 0; k < kSteps; ++k) {
+      cs[k] = 0;
+      if (k < steps) {
+        const int e = base0 + k * 64 + lane;
+        if (e < n_experts) cs[k] = load_count(counts, is_i64, e);
+      }
     }
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int base = base0 + k * 64;
-      if (base < n_experts) {  // wave-uniform
-        const int c = c4[k];
-        const int pc = (c + pad - 1) / pad * pad;
+    for (int k = 0; k < kSteps; ++k) {
+      if (k < steps) {
+        const int base = base0 + k * 64;
+        const int c = cs[k];
+        const int pc = (c + pad - 1) & -pad;  // pad is a power of two (1 or 16)
         const int nb = (c + kGroup - 1) / kGroup;
         const int rows = wave_inclusive_scan(pc);
         const int blocks = wave_inclusive_scan(nb);
