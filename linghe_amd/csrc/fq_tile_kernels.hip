@@ -13,7 +13,12 @@
 //   and the memory-side cache: gather+pad+quant 75 -> 55 us, RMSNorm+quant after the
 //   statistic pass 25 -> 21 us (8192 x 2048) and 146 -> 122 us (16384 x 7168).  The
 //   SwiGLU backward is 3-7 % slower when its transposed stores carry it, the plain
-//   blockwise quantisers 10-17 % slower with any of it.
+//   blockwise quantisers 10-17 % slower with any of it.  Transposed rows that do not start
+//   on 16-byte boundaries (M or a per-expert count that is not a multiple of 16) are where
+//   the hint on the transposed stores costs most: the SwiGLU forward takes 100 instead of
+//   70 us at 16300 x 3584 with it (and gains 3 % at 8192 x 2048), so it keeps the hint on
+//   the row-wise codes only; the RMSNorm tile kernel gains 18 % from it on aligned rows
+//   and loses 8 % on unaligned ones.
 //   FQ_LDNT_<kernel>: the bulk loads carry it (3-5 % on the SwiGLU kernels and the
 //   RMSNorm tile kernel, nothing on the plain quantisers).
 #ifndef FQ_NT_BLOCKWISE
@@ -23,7 +28,7 @@
 #define FQ_NT_PERMUTE 3
 #endif
 #ifndef FQ_NT_SILU_FWD
-#define FQ_NT_SILU_FWD 3
+#define FQ_NT_SILU_FWD 2
 #endif
 #ifndef FQ_NT_SILU_BWD
 #define FQ_NT_SILU_BWD 2
