@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256) void rowsum_kernel(const float* __restrict__ p
 // RMSNorm + quant on a tile with the row statistic given:
 //   y = (x * rstd[row]) * gamma[col]
 // ---------------------------------------------------------------------------
-template <int KIND, bool ROUND, int MODE>
+template <int KIND, bool ROUND, int MODE, int NT>
 __global__ __launch_bounds__(2048 / FQ_RPT_RMS) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
                                                                  const uint16_t* __restrict__ gamma,
                                                                  const float* __restrict__ rstd, OutPtrs out,
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(2048 / FQ_RPT_RMS) void rmsnorm_quant_tile_kernel(c
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[s][j] = (a[j] * r) * gm[j];
   }
-  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_RMSNORM>(v, make_out(out, g, n, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, NT>(v, make_out(out, g, n, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -400,11 +400,14 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
   const int64_t tiles = ((M + kGroup - 1) / kGroup) * (n / kGroup);
   if (tiles == 0) return hipSuccess;
   const dim3 grid((unsigned)tiles), block(2048 / FQ_RPT_RMS);
+  // transposed rows start every M bytes: off 16-byte boundaries their stores go out plain
+  const bool aligned_rows = M % 16 == 0;
   FQ_DISPATCH_KIND(kind, K,
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
-        hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD>), grid, block, 0, stream, (const uint16_t*)x,
-                           (const uint16_t*)gamma, rstd, out, M, n);)))
+        FQ_DISPATCH_BOOL(aligned_rows, A,
+          hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD, A ? FQ_NT_RMSNORM : (FQ_NT_RMSNORM & 2)>), grid,
+                             block, 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, rstd, out, M, n);))))
   return hipGetLastError();
 }
 
