@@ -208,7 +208,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   __shared__ TileShared<RPT> sh;
   const int nb = n / kGroup;
   const int64_t N = 2 * (int64_t)n;
-  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch);
+  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch, BATCHED);  // the per-expert form takes the XCD remap
   if (!g.valid) return;
   uint4 r1[RPT], r2[RPT], rgd[RPT];
   const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
@@ -282,11 +282,11 @@ template <int KIND, bool ROUND, int MODE, int NT>
 __global__ __launch_bounds__(2048 / FQ_RPT_RMS) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
                                                                  const uint16_t* __restrict__ gamma,
                                                                  const float* __restrict__ rstd, OutPtrs out,
-                                                                 int64_t M, int n) {
+                                                                 int64_t M, int n, int remap) {
   constexpr int RPT = FQ_RPT_RMS;
   __shared__ TileShared<RPT> sh;
   BatchArgs none{nullptr, 0, 0};
-  const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none);
+  const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none, remap != 0);
   if (!g.valid) return;
   uint4 raw[RPT];
   load_rows<RPT, FQ_LDNT_RMSNORM != 0>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
@@ -402,12 +402,15 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
   const dim3 grid((unsigned)tiles), block(2048 / FQ_RPT_RMS);
   // transposed rows start every M bytes: off 16-byte boundaries their stores go out plain
   const bool aligned_rows = M % 16 == 0;
+  // XCD remap (see resolve_tile): wide rows and several waves of workgroups
+  const int remap = aligned_rows && n >= 4096 && tiles >= 3072;
   FQ_DISPATCH_KIND(kind, K,
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
         FQ_DISPATCH_BOOL(aligned_rows, A,
           hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD, A ? FQ_NT_RMSNORM : (FQ_NT_RMSNORM & 2)>), grid,
-                             block, 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, rstd, out, M, n);))))
+                             block, 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, rstd, out, M, n,
+                             remap);))))
   return hipGetLastError();
 }
 
