@@ -20,6 +20,9 @@ namespace fq {
 // (-3 to -7 % with the hint on the RMSNorm backward, the bf16 SwiGLU rows and the
 // 128x128 block quantiser); FQ_ROW_LDNT puts the hint on the loads of rows that the
 // kernel reads once.
+#ifndef FQ_FWD_REMAP
+#define FQ_FWD_REMAP 1
+#endif
 #ifndef FQ_NT_ROWS
 #define FQ_NT_ROWS 1
 #endif
@@ -133,8 +136,17 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
   const int tid = threadIdx.x;
   uint4 gm[NCHUNK];
   load_row<T, NCHUNK>(gamma, n, gm);
-  const int64_t G = gridDim.x;  // rows blockIdx.x, +G, +2G, ...
-  const int64_t r0 = blockIdx.x;
+  const int64_t G = gridDim.x;  // rows b, b + G, b + 2G, ... with b the workgroup's logical index:
+  // workgroup i runs on XCD i % 8, and every XCD takes one contiguous eighth of the
+  // indices in the quantising form (3-7 % faster; the bf16 form is 8-20 % slower with it)
+  int64_t r0 = blockIdx.x;
+  if constexpr (OUT == 1 && FQ_FWD_REMAP != 0) {
+    const int Gi = (int)gridDim.x;
+    const int per = (Gi + 7) >> 3;
+    const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
+    const int full = (Gi & 7) ? (Gi & 7) : 8;
+    r0 = xcd < full ? xcd * per + slot : full * per + (xcd - full) * (per - 1) + slot;
+  }
   const int64_t r1 = M;
   (void)rows_per_wg;
   if (r0 >= r1) return;
