@@ -29,7 +29,6 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-SINGLE_PASS_CASES = {"cfg1_single", "cfg5b_single"}  # RMSNorm+quant mode 2 with the workspace (one pass over x)
 INFINITY_CACHE_BYTES = 256 << 20
 FP8 = torch.float8_e4m3fn
 
@@ -85,9 +84,8 @@ def build_cases(names, dev):
                 s["st"] = torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32)
             else:
                 s["qt"], s["st"] = None, None
-            ws, ws_bytes = _lib.norm_workspace(s["x"], M, n) if name in SINGLE_PASS_CASES else (None, 0)
             s["args"] = (_p(s["x"]), _p(gd), _p(s["q"]), _p(s["s"]), _p(s["rstd"]), _p(s["qt"]), _p(s["st"]),
-                         M, n, float(eps), 0, mode, _lib.FQ_E4M3, _p(ws), ws_bytes, stream)
+                         M, n, float(eps), 0, mode, _lib.FQ_E4M3, stream)
             return s
 
         def launch(s):
@@ -99,7 +97,7 @@ def build_cases(names, dev):
 
         label = "triton_rms_norm_and_block_quant_forward(output_mode=%d)" % mode
         if mode == 2:
-            label += " single pass" if name in SINGLE_PASS_CASES else " two passes"
+            label += " two passes"
         return Case(name, label, [M, n],
                     configs.bytes_rmsnorm_quant(M, n, mode), make_set, launch, cpu_fn)
 
@@ -111,9 +109,7 @@ def build_cases(names, dev):
         return lazy["cfg5"]
 
     add("cfg1", build=lambda: rms_quant_case("cfg1", configs.cfg1_rmsnorm_quant(), 2))
-    add("cfg1_single", build=lambda: rms_quant_case("cfg1_single", configs.cfg1_rmsnorm_quant(), 2))
     add("cfg5b", build=lambda: rms_quant_case("cfg5b", cfg5(), 2))
-    add("cfg5b_single", build=lambda: rms_quant_case("cfg5b_single", cfg5(), 2))
     add("cfg5c", build=lambda: rms_quant_case("cfg5c", cfg5(), 1))
 
     # ---------------------------------------------------------------- cfg2
@@ -459,7 +455,7 @@ def time_cpu(case, budget_s):
 # the difference is the second read of x.
 CFG1_MEASURED_TRAFFIC_BYTES = 102.48e6
 
-ALL = ["cfg1", "cfg1_single", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5b_single", "cfg5c",
+ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
        "next_permute",
        "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router"]
 

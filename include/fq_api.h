@@ -110,34 +110,15 @@ int64_t fq_rmsnorm_bwd_num_partials(int64_t M, int64_t n);
 int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx, float* dgamma,
                    float* dgamma_partials, int64_t n_partials, int64_t M, int64_t n, float eps, void* stream);
 
-/* bytes of device workspace fq_rmsnorm_quant_fwd uses for output_mode 2 */
-int64_t fq_rmsnorm_quant_workspace_bytes(int64_t M, int64_t n);
-
 /* triton_rms_norm_and_block_quant_forward, linghe/utils/norm.py:343-502.
  * mode 0: writes q, s, rstd.  mode 1: reads rstd, writes qt, st.
- * mode 2: writes q, s, rstd, qt, st.
- * workspace (mode 2 only, may be NULL): caller-owned device buffer of at least
- * fq_rmsnorm_quant_workspace_bytes(M, n) bytes, 256-byte aligned, ALL ZERO when
- * it is first handed to the library and written by nobody else afterwards.
- * With it x is read once: the workgroups of a 128-row slab exchange the row
- * statistic through it, every entry stamped with a per-call counter, so the
- * buffer needs no clearing between calls and can be shared by calls of any
- * shape on one stream (calls that may overlap in time need a buffer each; clear
- * it again after 2^32 calls).  The workgroups of the single pass wait for each
- * other, so it wants the GPU to itself; every wait is bounded
- * (fq_set_wait_limit) and a workgroup that gives up recomputes what it waited
- * for, so results never depend on timing.  Without a workspace, or while
- * `stream` is being captured into a graph (a replay would repeat the stamp),
- * mode 2 runs as two passes - the row statistic, then the tile kernel - and
- * reads x twice; that is the faster variant at every size measured so far. */
+ * mode 2: writes q, s, rstd, qt, st; runs as two launches on `stream` - the
+ * row statistic (x read once, rstd written), then the 128x128 tile kernel that
+ * reads x again (the second read is served by the memory-side cache when x fits
+ * it) and emits both layouts. */
 int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt, float* st,
                          int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
-                         void* workspace, int64_t workspace_bytes, void* stream);
-
-/* Upper bound on the polls a workgroup of the single-pass RMSNorm kernel spends
- * waiting for its slab's statistic before it computes the statistic itself
- * (<= 0 restores the default).  Process-wide; meant for tests of that path. */
-void fq_set_wait_limit(int polls);
+                         void* stream);
 
 /* triton_rms_norm_fp32_gemm_block_quant_forward, output_mode 0,
  * linghe/utils/norm.py:690-784 (kernel :616-687).  x bf16 [M,K], gamma bf16 [K],

@@ -34,15 +34,14 @@ SIGNATURES = {
     "fq_group_quant": [_P, _P, _P, _L, _L, _I, _I, _P],
     "fq_rmsnorm_fwd": [_P, _P, _P, _P, _L, _L, _F, _I, _P],
     "fq_rmsnorm_bwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _P],
-    "fq_rmsnorm_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _I, _I, _P, _L, _P],
+    "fq_rmsnorm_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _I, _I, _P],
     "fq_rmsnorm_router_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _I, _P],
     "fq_swiglu_quant_fwd": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_swiglu_quant_bwd": [_P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_swiglu_quant_fwd": [_P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_swiglu_quant_bwd": [_P, _P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
 }
-OTHER_SYMBOLS = ["fq_version", "fq_last_error", "fq_rmsnorm_bwd_num_partials",
-                 "fq_rmsnorm_quant_workspace_bytes", "fq_set_wait_limit"]
+OTHER_SYMBOLS = ["fq_version", "fq_last_error", "fq_rmsnorm_bwd_num_partials"]
 
 
 def _load() -> ctypes.CDLL:
@@ -61,10 +60,6 @@ def _load() -> ctypes.CDLL:
     lib.fq_last_error.restype = ctypes.c_char_p
     lib.fq_rmsnorm_bwd_num_partials.argtypes = [_L, _L]
     lib.fq_rmsnorm_bwd_num_partials.restype = _L
-    lib.fq_rmsnorm_quant_workspace_bytes.argtypes = [_L, _L]
-    lib.fq_rmsnorm_quant_workspace_bytes.restype = _L
-    lib.fq_set_wait_limit.argtypes = [_I]
-    lib.fq_set_wait_limit.restype = None
     return lib
 
 
@@ -124,22 +119,3 @@ def require_device_bf16(t: torch.Tensor, name: str) -> None:
         raise RuntimeError(f"{name} must live on the GPU: the HIP kernels are the only implementation")
     if t.dtype != torch.bfloat16:
         raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
-
-
-# ---------------------------------------------------------------------------
-# device workspace of the single-pass RMSNorm+quant kernel: one zero-initialised
-# buffer per (device, stream), grown on demand.  Entries are stamped per call,
-# so the buffer is never cleared again.
-# ---------------------------------------------------------------------------
-_norm_workspaces = {}
-
-
-def norm_workspace(t: torch.Tensor, M: int, n: int):
-    """-> (workspace tensor, bytes needed)"""
-    need = int(lib.fq_rmsnorm_quant_workspace_bytes(M, n))
-    key = (t.device.index, stream_of(t))
-    buf = _norm_workspaces.get(key)
-    if buf is None or buf.numel() < need:
-        buf = torch.zeros(max(2 * need, 1 << 20), dtype=torch.uint8, device=t.device)
-        _norm_workspaces[key] = buf
-    return buf, need

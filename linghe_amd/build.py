@@ -2,7 +2,7 @@
 
     python -m linghe_amd.build
 
-hipcc cross-compiles for gfx950 without a GPU.  The three translation units are
+hipcc cross-compiles for gfx950 without a GPU.  The translation units are
 compiled in parallel and linked into ``linghe_amd/libfq_gfx950.so``.
 """
 from __future__ import annotations
@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libfq_gfx950.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["fq_api.hip", "fq_tile_kernels.hip", "fq_row_kernels.hip", "fq_norm_fused.hip", "fq_router.hip"]
+SOURCES = ["fq_api.hip", "fq_tile_kernels.hip", "fq_row_kernels.hip", "fq_router.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -1,11 +1,9 @@
 // C-ABI layer: argument validation + dispatch to the kernel launchers.
-// Holds no mutable global state besides the per-thread error message.
+// The only mutable state is the per-thread error message.
 #include "../../include/fq_api.h"
 
 #include <stdarg.h>
 #include <stdio.h>
-
-#include <atomic>
 
 #include "fq_launch.h"
 
@@ -164,11 +162,11 @@ int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float
   const char* fn = "fq_rmsnorm_bwd";
   int rc = check_norm_shape(fn, M, n);
   if (rc) return rc;
-  FQ_REQUIRE(dgamma && dgamma_partials, FQ_ERR_ARG, "%s: dgamma outputs are NULL", fn);
+  FQ_REQUIRE(dgamma, FQ_ERR_ARG, "%s: dgamma is NULL", fn);
   FQ_REQUIRE(n_partials == fq::rmsnorm_bwd_partials(M), FQ_ERR_SHAPE,
              "%s: n_partials must equal fq_rmsnorm_bwd_num_partials(M, n)", fn);
-  if (M > 0) {
-    FQ_REQUIRE(dy && x && gamma && dx, FQ_ERR_ARG, "%s: NULL pointer", fn);
+  if (M > 0) {  // with no rows only dgamma is touched (it is zeroed); the row kernel is not launched
+    FQ_REQUIRE(dy && x && gamma && dx && dgamma_partials, FQ_ERR_ARG, "%s: NULL pointer", fn);
     FQ_REQUIRE(aligned16(dy) && aligned16(x) && aligned16(gamma) && aligned16(dx) && aligned16(dgamma_partials),
                FQ_ERR_ARG, "%s: misaligned pointer", fn);
   }
@@ -177,26 +175,9 @@ int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float
                       fn);
 }
 
-int64_t fq_rmsnorm_quant_workspace_bytes(int64_t M, int64_t n) {
-  if (M <= 0 || n <= 0 || n % 128 != 0 || n > 8192) return 0;
-  return fq::rmsnorm_fused_scratch_bytes(M, (int)n);
-}
-
-// stamp of the next single-pass launch (never 0: a cleared workspace reads as "not ready")
-static std::atomic<uint32_t> g_stamp{0};
-static uint32_t next_stamp() {
-  uint32_t t;
-  do { t = g_stamp.fetch_add(1u) + 1u; } while (t == 0u);
-  return t;
-}
-
-static std::atomic<int> g_wait_limit{0};
-
-void fq_set_wait_limit(int polls) { g_wait_limit.store(polls > 0 ? polls : 0); }
-
 int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt, float* st,
                          int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
-                         void* workspace, int64_t workspace_bytes, void* stream) {
+                         void* stream) {
   const char* fn = "fq_rmsnorm_quant_fwd";
   int rc = check_common(fn, M, n, round_scale, fp8_kind);
   if (rc) return rc;
@@ -207,27 +188,6 @@ int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, fl
   FQ_REQUIRE(aligned16(x) && aligned16(gamma), FQ_ERR_ARG, "%s: misaligned pointer", fn);
   hipStream_t st_ = (hipStream_t)stream;
   if ((rc = check_tiles(fn, ((M + 127) / 128) * (n / 128)))) return rc;
-  // single pass only when the caller brings the exchange workspace
-  bool single_pass = output_mode == 2 && workspace != nullptr;
-  if (single_pass) {
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st_, &cap) != hipSuccess) {
-      (void)hipGetLastError();
-      cap = hipStreamCaptureStatusNone;
-    }
-    if (cap != hipStreamCaptureStatusNone) single_pass = false;  // a replay would reuse the stamp
-  }
-  if (single_pass) {
-    FQ_REQUIRE(workspace_bytes >= fq::rmsnorm_fused_scratch_bytes(M, (int)n), FQ_ERR_ARG,
-               "%s: workspace of %lld bytes is smaller than fq_rmsnorm_quant_workspace_bytes", fn,
-               (long long)workspace_bytes);
-    FQ_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FQ_ERR_ARG,
-               "%s: workspace must be 256-byte aligned", fn);
-    return check_launch(fq::launch_rmsnorm_quant_fused(x, gamma, q, s, rstd, qt, st, workspace, next_stamp(), M,
-                                                       (int)n, eps, round_scale, 2, fp8_kind, g_wait_limit.load(),
-                                                       st_),
-                        fn);
-  }
   if (output_mode == 0) {
     return check_launch(fq::launch_rmsnorm_fwd(x, gamma, q, s, rstd, M, (int)n, eps, 0, 1, round_scale, fp8_kind, st_),
                         fn);

@@ -30,12 +30,6 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
                                      void* qt, float* st, int64_t M, int n, int round_scale, int mode, int kind,
                                      hipStream_t stream);
 
-int64_t rmsnorm_fused_scratch_bytes(int64_t M, int n);
-
-hipError_t launch_rmsnorm_quant_fused(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt,
-                                      float* st, void* scratch_ws, uint32_t tag, int64_t M, int n, float eps,
-                                      int round_scale, int mode, int kind, int wait_limit, hipStream_t stream);
-
 hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float* scale, float* rstd, int64_t M,
                               int n, float eps, int reuse_rstd, int quant, int round_scale, int kind,
                               hipStream_t stream);

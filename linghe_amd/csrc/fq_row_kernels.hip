@@ -599,6 +599,10 @@ int64_t rmsnorm_bwd_partials(int64_t M) {
 hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
                               float* dgamma, float* dg_part, int64_t n_partials, int64_t M, int n, float eps,
                               hipStream_t stream) {
+  if (M == 0) {  // no rows: dgamma = 0, and no kernel touches dy, x, gamma or dx
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((n + 63) / 64)), dim3(1024), 0, stream, dg_part, dgamma, 0, n);
+    return hipGetLastError();
+  }
   const int64_t P = n_partials;
   const int rows_per_wg = (int)((M + P - 1) / P);
   const dim3 grid((unsigned)P);

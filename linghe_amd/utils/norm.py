@@ -13,14 +13,6 @@ from .. import _lib
 
 _MAX_HIDDEN = 8192  # the reference asserts next_power_of_2(n) <= 8192
 
-# output_mode 2 of triton_rms_norm_and_block_quant_forward:
-#   False  two passes (row statistic, then the tile kernel): the fastest measured
-#          variant on MI355X at every size tried;
-#   True   hand the library its workspace, so that the call is ONE pass over x (the
-#          statistic is exchanged between workgroups inside the kernel):
-#          algorithmic HBM traffic, 45-60 % slower at the sizes measured.
-SINGLE_PASS = False
-
 
 def _rows_cols(x):
     shape = x.shape
@@ -153,16 +145,12 @@ def triton_rms_norm_and_block_quant_forward(
 
     if M > 0:
         with _lib.on_device(device):
-            ws, ws_bytes = (None, 0)
-            if output_mode == 2 and SINGLE_PASS:
-                ws, ws_bytes = _lib.norm_workspace(x, M, n)
             _lib.check(_lib.lib.fq_rmsnorm_quant_fwd(
                 _lib.ptr(x), _lib.ptr(weight),
                 _lib.ptr(out) if output_mode != 1 else None,
                 _lib.ptr(scale) if output_mode != 1 else None,
                 _lib.ptr(rms), _lib.ptr(transpose_output), _lib.ptr(transpose_scale),
-                M, n, float(eps), int(bool(round_scale)), output_mode, kind,
-                _lib.ptr(ws), ws_bytes, _lib.stream_of(x)))
+                M, n, float(eps), int(bool(round_scale)), output_mode, kind, _lib.stream_of(x)))
     return out, scale, rms, transpose_output, transpose_scale
 
 
@@ -230,5 +218,5 @@ def triton_rms_norm_fp32_gemm_block_quant_forward(
         else:
             _lib.check(_lib.lib.fq_rmsnorm_quant_fwd(
                 _lib.ptr(x), _lib.ptr(norm_weight), None, None, _lib.ptr(rms), _lib.ptr(xt_q), _lib.ptr(xt_s),
-                M, K, float(eps), int(bool(round_scale)), 1, _lib.FQ_E4M3, None, 0, _lib.stream_of(x)))
+                M, K, float(eps), int(bool(round_scale)), 1, _lib.FQ_E4M3, _lib.stream_of(x)))
     return y, rms, logits, x_q, x_s, xt_q, xt_s

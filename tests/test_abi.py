@@ -32,15 +32,30 @@ def test_library_exports_every_declared_symbol():
     assert _lib.lib.fq_version() >= 100
 
 
-def test_argument_counts_match_header():
+def _ctype_of(decl: str):
+    """C parameter declaration -> the ctypes type a binding must use for it."""
+    decl = decl.strip()
+    if "*" in decl:
+        return ctypes.c_void_p
+    words = [w for w in re.split(r"\s+", decl) if w not in ("const",)]
+    base = " ".join(words[:-1])  # drop the parameter name
+    return {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "float": ctypes.c_float}[base]
+
+
+def test_argument_types_match_header():
+    """Every bound signature agrees with its declaration type by type: a pointer is a
+    void pointer, int / int64_t / float map to the ctypes of the same width."""
     from linghe_amd import _lib
 
     text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
     for name, argtypes in _lib.SIGNATURES.items():
-        m = re.search(r"\b" + name + r"\s*\((.*?)\)\s*;", text, flags=re.S)
+        m = re.search(r"\bint\s+" + name + r"\s*\((.*?)\)\s*;", text, flags=re.S)
         assert m, name
-        n_args = len([a for a in m.group(1).split(",") if a.strip()])
-        assert n_args == len(argtypes), (name, n_args, len(argtypes))
+        declared = [_ctype_of(a) for a in m.group(1).split(",") if a.strip()]
+        assert declared == list(argtypes), (name, declared, argtypes)
+    m = re.search(r"\bint64_t\s+fq_rmsnorm_bwd_num_partials\s*\((.*?)\)\s*;", text, flags=re.S)
+    assert [_ctype_of(a) for a in m.group(1).split(",")] == list(_lib.lib.fq_rmsnorm_bwd_num_partials.argtypes)
+    assert _lib.lib.fq_rmsnorm_bwd_num_partials.restype is ctypes.c_int64
 
 
 def test_c_side_validation_without_gpu():
@@ -83,6 +98,19 @@ def test_c_side_validation_without_gpu():
     # bf16 SwiGLU: weight and dw go together
     rc = L.fq_swiglu_bwd(None, None, None, 0, None, ctypes.c_void_p(16), 16, 128, None)
     assert rc == -1
+    # RMSNorm backward: a wrong partial count is refused before anything else is looked at,
+    # and with rows present every pointer must be there (no launch with a NULL gamma)
+    n_part = L.fq_rmsnorm_bwd_num_partials(64, 256)
+    rc = L.fq_rmsnorm_bwd(None, None, None, None, None, ctypes.c_void_p(256), ctypes.c_void_p(256), n_part + 1, 64,
+                          256, 1e-6, None)
+    assert rc == -2
+    rc = L.fq_rmsnorm_bwd(ctypes.c_void_p(256), ctypes.c_void_p(256), None, None, ctypes.c_void_p(256),
+                          ctypes.c_void_p(256), ctypes.c_void_p(256), n_part, 64, 256, 1e-6, None)
+    assert rc == -1 and b"NULL" in L.fq_last_error()
+    # ... and with no rows a NULL dgamma is still refused (it is the one output that is written)
+    rc = L.fq_rmsnorm_bwd(None, None, None, None, None, None, None, L.fq_rmsnorm_bwd_num_partials(0, 256), 0, 256,
+                          1e-6, None)
+    assert rc == -1 and b"dgamma" in L.fq_last_error()
     # empty problem is a no-op
     assert L.fq_group_quant(None, None, None, 0, 128, 0, 0, None) == 0
     assert L.fq_swiglu_fwd(None, None, 0, None, 0, 128, None) == 0

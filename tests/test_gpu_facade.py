@@ -210,9 +210,7 @@ def test_block_batch_weighted_silu(gpu, is_recomputing):
 def test_entry_points_under_graph_capture(gpu):
     """The library only enqueues work on the given stream, so its calls can be
     captured into a graph: every replay (with eager work and synchronisations in
-    between) must reproduce the eager results bit for bit.  With the single-pass
-    switch on, a capturing stream still gets the two-pass kernels."""
-    import linghe_amd.utils.norm as norm_mod
+    between) must reproduce the eager results bit for bit."""
     from linghe_amd.quant.block import triton_blockwise_quant
     from linghe_amd.utils.norm import triton_rms_norm_and_block_quant_forward, triton_rms_norm_backward
     from linghe_amd.utils.silu import (triton_batch_weighted_silu_and_block_quant_forward,
@@ -243,18 +241,14 @@ def test_entry_points_under_graph_capture(gpu):
     eager1, eager2 = bits(run(x)), bits(run(x2))
     torch.cuda.synchronize()
     static_in = x.clone()
-    norm_mod.SINGLE_PASS = True
-    try:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            run(static_in)  # warm-up on the capture stream
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            outs = run(static_in)
-    finally:
-        norm_mod.SINGLE_PASS = False
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(static_in)  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = run(static_in)
     for rep, (src, want) in enumerate(((x, eager1), (x2, eager2), (x, eager1), (x2, eager2))):
         static_in.copy_(src)
         graph.replay()

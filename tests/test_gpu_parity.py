@@ -230,107 +230,6 @@ def test_rmsnorm_and_block_quant(gpu, M, N, round_scale):
     p_ref = O.rms_norm_and_block_quant_forward(x, w, round_scale=round_scale, rstd=rms2.cpu())
     check_quant_pair("rms.pinned.row", p_ref[0], p_ref[1], q2, s2, **EXACT)
     check_quant_pair("rms.pinned.col", p_ref[3], p_ref[4], qt2, st2, **EXACT)
-    # single-pass variant (opt-in): same rule; repeated calls reuse the workspace
-    # (entries are stamped per call, nothing is cleared)
-    import linghe_amd.utils.norm as norm_mod
-    norm_mod.SINGLE_PASS = True
-    try:
-        q3, s3, rms3, qt3, st3 = fwd(xd, wd, round_scale=round_scale, output_mode=2)
-        q4, s4, rms4, qt4, st4 = fwd(xd, wd, round_scale=round_scale, output_mode=2)
-        torch.cuda.synchronize()
-    finally:
-        norm_mod.SINGLE_PASS = False
-    C.assert_scales(r_ref, rms3.cpu(), "rstd (single pass)", max_ulp=4, min_within_1ulp=0.9)
-    p_ref = O.rms_norm_and_block_quant_forward(x, w, round_scale=round_scale, rstd=rms3.cpu())
-    check_quant_pair("rms.single.row", p_ref[0], p_ref[1], q3, s3, **EXACT)
-    check_quant_pair("rms.single.col", p_ref[3], p_ref[4], qt3, st3, **EXACT)
-    for a, b in ((q3, q4), (s3, s4), (rms3, rms4), (qt3, qt4), (st3, st4)):
-        assert torch.equal(a.view(torch.uint8).cpu(), b.view(torch.uint8).cpu())
-
-
-def test_rmsnorm_quant_single_pass_wait_bound(gpu):
-    """The single-pass kernel's wait for the slab statistic is bounded: with the
-    bound forced to one poll most workgroups give up and recompute the statistic
-    themselves; every output must be bit-identical to the normal run, and the
-    workspace must still be reusable afterwards.  A NULL workspace selects the
-    two-pass path, whose codes must agree to the usual rule."""
-    from linghe_amd import _lib
-    from linghe_amd.utils.norm import triton_rms_norm_and_block_quant_forward as fwd
-
-    announce("rmsnorm+quant single pass, forced short wait")
-    g = gen(23)
-    M, N = 1000, 2048
-    x = randn_bf16(g, M, N)
-    w = gamma_bf16(g, N)
-    xd, wd = _dev(x, gpu), _dev(w, gpu)
-    import linghe_amd.utils.norm as norm_mod
-    norm_mod.SINGLE_PASS = True
-    try:
-        base = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
-        torch.cuda.synchronize()
-        try:
-            _lib.lib.fq_set_wait_limit(1)
-            short = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
-            torch.cuda.synchronize()
-        finally:
-            _lib.lib.fq_set_wait_limit(0)
-        again = [t.view(torch.uint8).cpu() if t.dtype != torch.float32 else t.cpu() for t in fwd(xd, wd)]
-        torch.cuda.synchronize()
-    finally:
-        norm_mod.SINGLE_PASS = False
-    for a, b, c in zip(base, short, again):
-        assert torch.equal(a, b) and torch.equal(a, c)
-    # two-pass path through the C ABI (no workspace)
-    q = torch.empty((M, N), device=gpu, dtype=E4M3)
-    s = torch.empty((N // 128, M), device=gpu, dtype=torch.float32)
-    r = torch.empty((M,), device=gpu, dtype=torch.float32)
-    qt = torch.empty((N, M), device=gpu, dtype=E4M3)
-    st = torch.empty(((M + 127) // 128, N), device=gpu, dtype=torch.float32)
-    _lib.check(_lib.lib.fq_rmsnorm_quant_fwd(xd.data_ptr(), wd.data_ptr(), q.data_ptr(), s.data_ptr(), r.data_ptr(),
-                                             qt.data_ptr(), st.data_ptr(), M, N, 1e-6, 0, 2, 0, None, 0,
-                                             _lib.stream_of(xd)))
-    torch.cuda.synchronize()
-    ref = O.rms_norm_and_block_quant_forward(x, w, rstd=r.cpu())
-    check_quant_pair("rms.two_pass.row", ref[0], ref[1], q, s, **EXACT)
-    check_quant_pair("rms.two_pass.col", ref[3], ref[4], qt, st, **EXACT)
-
-
-@pytest.mark.parametrize("M,N", [(8192, 2048), (4096 + 40, 7168), (16384, 512), (3000, 1536)])
-@pytest.mark.parametrize("short_wait", [False, True])
-def test_rmsnorm_quant_single_pass_many_steps(gpu, M, N, short_wait):
-    """Shapes with more tiles than the device holds workgroups: every workgroup of
-    the single-pass kernel walks several tiles.  Its outputs, statistic included,
-    must equal the two-pass path bit for bit (both add the same exact group sums),
-    also when every wait is cut to one poll and the workgroups fall back to
-    recomputing the statistic in the middle of their sequence."""
-    from linghe_amd import _lib
-    from linghe_amd.utils.norm import triton_rms_norm_and_block_quant_forward as fwd
-    import linghe_amd.utils.norm as norm_mod
-
-    announce("rmsnorm+quant single pass, many steps", M, N, short_wait)
-    g = gen(29)
-    x = randn_bf16(g, M, N, scale=2.0)
-    w = gamma_bf16(g, N)
-    xd, wd = _dev(x, gpu), _dev(w, gpu)
-    two = fwd(xd, wd, round_scale=False, output_mode=2)
-    torch.cuda.synchronize()
-    norm_mod.SINGLE_PASS = True
-    try:
-        if short_wait:
-            _lib.lib.fq_set_wait_limit(1)
-        one = fwd(xd, wd, round_scale=False, output_mode=2)
-        again = fwd(xd, wd, round_scale=False, output_mode=2)
-        torch.cuda.synchronize()
-    finally:
-        _lib.lib.fq_set_wait_limit(0)
-        norm_mod.SINGLE_PASS = False
-    names = ("q", "s", "rstd", "qt", "st")
-    for name, a, b, c in zip(names, two, one, again):
-        av, bv, cv = (t.view(torch.uint8).cpu() for t in (a, b, c))
-        assert torch.equal(av, bv), f"{name}: single pass differs from two passes"
-        assert torch.equal(bv, cv), f"{name}: second single-pass call differs"
-    ref = O.rms_norm_and_block_quant_forward(x[:256], w, rstd=one[2][:256].cpu())
-    check_quant_pair("rms.single.steps.row", ref[0], ref[1], one[0][:256], one[1][:, :256], **EXACT)
 
 
 # ------------------------------------------------------------------ SwiGLU
