@@ -1,4 +1,9 @@
-"""Autograd callers of the SwiGLU+quant path (reference: linghe/facade/silu.py:11-170)."""
+"""Autograd callers of the SwiGLU + quantisation path (contract:
+linghe/facade/silu.py:11-170): the dense form on a [s, b, 2h] activation and the
+per-expert weighted form on [tokens, 2h].  Forward and backward both return the
+caller's quantised-tensor class; the backward's codes are in the FP8 format of the
+gradient quantizer.
+"""
 import torch
 
 from ..utils.silu import (
@@ -7,66 +12,34 @@ from ..utils.silu import (
     triton_silu_and_block_quant_backward,
     triton_silu_and_block_quant_forward,
 )
-
-
-def _mode_of(is_recomputing):
-    if is_recomputing is None:
-        return 2
-    return 1 if is_recomputing else 0
+from ._qtensor import Codes, Folded, kernel_fp8_dtype, output_mode, wrap
 
 
 class BlockSiluFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, quantizer, grad_quantizer, cls):
-        shape = input.shape
-        assert len(shape) == 3
-        rows, half = shape[0] * shape[1], shape[2] // 2
-        ctx.grad_quantizer = grad_quantizer
-        ctx.input_requires_grad = input.requires_grad
-        ctx.shape = shape
-        ctx.cls = cls
+        assert input.dim() == 3
+        act = Folded(input)
+        half = act.shape[-1] // 2
         ctx.save_for_backward(input)
-        x_q, x_scale, xt_q, xt_scale = triton_silu_and_block_quant_forward(
-            input.view(rows, shape[2]), round_scale=quantizer.force_pow_2_scales
-        )
-        out_shape = (shape[0], shape[1], half)
-        return cls(
-            shape=out_shape,
-            dtype=input.dtype,
-            fp8_dtype=quantizer.dtype,
-            rowwise_data=x_q.view(out_shape),
-            rowwise_scale_inv=x_scale,
-            columnwise_data=xt_q.view(half, shape[0], shape[1]),
-            columnwise_scale_inv=xt_scale,
-            quantizer=quantizer,
-            requires_grad=input.requires_grad,
-            is_2D_scaled=False,
-        )
+        ctx.sidecar = (grad_quantizer, cls, input.requires_grad)
+        got = triton_silu_and_block_quant_forward(
+            act.matrix(input), round_scale=quantizer.force_pow_2_scales,
+            fp8_dtype=kernel_fp8_dtype(quantizer.dtype))
+        return wrap(cls, act.unfold(Codes(*got), half), shape=(*act.lead, half), dtype=input.dtype,
+                    quantizer=quantizer, fp8_tag=quantizer.dtype, requires_grad=input.requires_grad)
 
     @staticmethod
     def backward(ctx, grad_output):
-        gshape = grad_output.shape
-        rows = gshape[0] * gshape[1]
         (input,) = ctx.saved_tensors
-        gq = ctx.grad_quantizer
-        x_q, x_scale, xt_q, xt_scale = triton_silu_and_block_quant_backward(
-            grad_output.contiguous().view(rows, gshape[2]),
-            input.view(rows, gshape[2] * 2),
-            round_scale=gq.force_pow_2_scales,
-        )
-        output = ctx.cls(
-            shape=ctx.shape,
-            dtype=grad_output.dtype,
-            fp8_dtype=gq.dtype,
-            rowwise_data=x_q.view(ctx.shape),
-            rowwise_scale_inv=x_scale,
-            columnwise_data=xt_q.view(ctx.shape[2], gshape[0], gshape[1]),
-            columnwise_scale_inv=xt_scale,
-            quantizer=gq,
-            requires_grad=ctx.input_requires_grad,
-            is_2D_scaled=False,
-        )
-        return output, None, None, None
+        grad_quantizer, cls, needs_grad = ctx.sidecar
+        act = Folded(input)
+        got = triton_silu_and_block_quant_backward(
+            act.matrix(grad_output.contiguous()), act.matrix(input),
+            round_scale=grad_quantizer.force_pow_2_scales, fp8_dtype=kernel_fp8_dtype(grad_quantizer.dtype))
+        dx = wrap(cls, act.unfold(Codes(*got), act.shape[-1]), shape=act.shape, dtype=grad_output.dtype,
+                  quantizer=grad_quantizer, fp8_tag=grad_quantizer.dtype, requires_grad=needs_grad)
+        return dx, None, None, None
 
 
 def block_silu_impl(input, quantizer, grad_quantizer, cls):
@@ -74,66 +47,40 @@ def block_silu_impl(input, quantizer, grad_quantizer, cls):
 
 
 class BlockBatchWeightedSiluFunction(torch.autograd.Function):
+    """Per-expert form: rows of `input` are grouped by expert (`counts` on the device,
+    `splits` the same numbers on the host), `weights` is one router probability per
+    row.  Outputs keep the kernels' per-expert packing, so nothing is re-viewed.
+    The quantizer lists are passed through to the tensor class; their first member
+    gives the scale rounding and the FP8 format of all experts."""
+
     @staticmethod
     def forward(ctx, input, weights, counts, splits, quantizers, grad_quantizers, cls, is_recomputing):
-        ctx.grad_quantizers = grad_quantizers
-        ctx.input_requires_grad = input.requires_grad
-        ctx.shape = input.shape
-        ctx.splits = splits
-        ctx.cls = cls
+        lead = quantizers[0]
         ctx.save_for_backward(input, weights, counts)
-        x_q, x_scale, xt_q, xt_scale = triton_batch_weighted_silu_and_block_quant_forward(
-            input,
-            weights,
-            counts,
-            splits=splits,
-            round_scale=quantizers[0].force_pow_2_scales,
-            output_mode=_mode_of(is_recomputing),
-        )
-        return cls(
-            shape=x_q.shape,
-            dtype=input.dtype,
-            fp8_dtype=quantizers[0].dtype,
-            rowwise_data=x_q,
-            rowwise_scale_inv=x_scale,
-            columnwise_data=xt_q,
-            columnwise_scale_inv=xt_scale,
-            quantizer=quantizers,
-            requires_grad=input.requires_grad,
-            is_2D_scaled=False,
-        )
+        ctx.sidecar = (splits, grad_quantizers, cls, input.requires_grad)
+        got = triton_batch_weighted_silu_and_block_quant_forward(
+            input, weights, counts, splits=splits, round_scale=lead.force_pow_2_scales,
+            output_mode=output_mode(is_recomputing), fp8_dtype=kernel_fp8_dtype(lead.dtype))
+        codes = Codes(*got)
+        return wrap(cls, codes, shape=codes.row.shape, dtype=input.dtype, quantizer=quantizers,
+                    fp8_tag=lead.dtype, requires_grad=input.requires_grad)
 
     @staticmethod
     def backward(ctx, grad_output):
         input, weights, counts = ctx.saved_tensors
-        gqs = ctx.grad_quantizers
-        x_q, x_scale, wgrad, xt_q, xt_scale = triton_batch_weighted_silu_and_block_quant_backward(
-            grad_output.contiguous(),
-            input,
-            weights,
-            counts,
-            splits=ctx.splits,
-            round_scale=gqs[0].force_pow_2_scales,
-        )
-        output = ctx.cls(
-            shape=ctx.shape,
-            dtype=grad_output.dtype,
-            fp8_dtype=gqs[0].dtype,
-            rowwise_data=x_q,
-            rowwise_scale_inv=x_scale,
-            columnwise_data=xt_q,
-            columnwise_scale_inv=xt_scale,
-            quantizer=gqs,
-            requires_grad=ctx.input_requires_grad,
-            is_2D_scaled=False,
-        )
-        return output, wgrad, None, None, None, None, None, None
+        splits, grad_quantizers, cls, needs_grad = ctx.sidecar
+        lead = grad_quantizers[0]
+        dq, dq_scale, dweights, dqt, dqt_scale = triton_batch_weighted_silu_and_block_quant_backward(
+            grad_output.contiguous(), input, weights, counts, splits=splits,
+            round_scale=lead.force_pow_2_scales, fp8_dtype=kernel_fp8_dtype(lead.dtype))
+        dx = wrap(cls, Codes(dq, dq_scale, dqt, dqt_scale), shape=input.shape, dtype=grad_output.dtype,
+                  quantizer=grad_quantizers, fp8_tag=lead.dtype, requires_grad=needs_grad)
+        # one gradient slot per forward argument: input, weights, then six non-tensors
+        return (dx, dweights) + (None,) * 6
 
 
-def block_batch_weighted_silu_impl(
-    input, weights, counts, splits, quantizers, grad_quantizers, cls, is_recomputing=None
-):
+def block_batch_weighted_silu_impl(input, weights, counts, splits, quantizers, grad_quantizers, cls,
+                                   is_recomputing=None):
     assert input.ndim == 2
-    return BlockBatchWeightedSiluFunction.apply(
-        input, weights, counts, splits, quantizers, grad_quantizers, cls, is_recomputing
-    )
+    return BlockBatchWeightedSiluFunction.apply(input, weights, counts, splits, quantizers, grad_quantizers,
+                                                cls, is_recomputing)

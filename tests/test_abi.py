@@ -192,3 +192,33 @@ def test_host_asserts_fire_on_cpu_tensors():
         triton_silu_and_block_quant_backward(torch.zeros(32, 128, dtype=torch.bfloat16).cuda()
                                              if torch.cuda.is_available() else
                                              torch.zeros(32, 128, dtype=torch.bfloat16), x)
+
+
+def test_facade_contract_helpers():
+    """The caller contract the autograd classes share (reference linghe/facade/norm.py:55-60,
+    facade/silu.py:43-65): recompute flag -> output mode, and the quantizer's dtype tag ->
+    the FP8 format the kernels are asked for."""
+    import torch
+
+    from linghe_amd.facade._qtensor import Codes, Folded, kernel_fp8_dtype, output_mode
+
+    assert [output_mode(v) for v in (None, False, True)] == [2, 0, 1]
+    assert kernel_fp8_dtype(torch.float8_e5m2) is torch.float8_e5m2
+    assert kernel_fp8_dtype(torch.float8_e4m3fn) is torch.float8_e4m3fn
+
+    class Tag:
+        def __init__(self, name):
+            self.name = name
+
+    assert kernel_fp8_dtype(Tag("kFloat8E5M2")) is torch.float8_e5m2
+    assert kernel_fp8_dtype(Tag("kFloat8E4M3")) is torch.float8_e4m3fn
+    with pytest.raises(TypeError):
+        kernel_fp8_dtype(torch.bfloat16)
+    with pytest.raises(TypeError):
+        kernel_fp8_dtype(Tag("kInt8"))
+    act = Folded(torch.zeros(6, 5, 256))
+    assert act.rows == 30 and act.matrix(torch.zeros(6, 5, 128)).shape == (30, 128)
+    codes = act.unfold(Codes(torch.zeros(30, 128), None, torch.zeros(128, 30), None), 128)
+    assert codes.row.shape == (6, 5, 128) and codes.col.shape == (128, 6, 5) and codes.row_scale is None
+    none = act.unfold(Codes(None, None, None, None), 128)
+    assert none.row is None and none.col is None

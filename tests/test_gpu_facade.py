@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from oracle import fq_oracle as O
-from tests.helpers import E4M3, announce, check_quant_pair, gamma_bf16, gen, randn_bf16
+from tests.helpers import E4M3, E5M2, announce, check_quant_pair, gamma_bf16, gen, randn_bf16
 from tests.test_gpu_parity import FUSED, FUSED_BWD, FUSED_NORM, check_bf16
 
 pytestmark = pytest.mark.gpu
@@ -127,11 +127,21 @@ def test_block_rms_norm(gpu, is_recomputing, pow2):
     torch.testing.assert_close(wd.grad.float().cpu(), dw_ref, rtol=1e-2, atol=1e-2 * float(dw_ref.abs().max()))
 
 
+class TEDType:
+    """stands in for TransformerEngine's DType enum members (matched by name)"""
+
+    def __init__(self, name):
+        self.name = name
+
+
 @pytest.mark.parametrize("pow2", [False, True])
-def test_block_silu(gpu, pow2):
+@pytest.mark.parametrize("gdtype,gtag", [(E4M3, E4M3), (E5M2, E5M2), (E5M2, TEDType("kFloat8E5M2"))])
+def test_block_silu(gpu, pow2, gdtype, gtag):
+    """The backward's codes are in the gradient quantizer's FP8 format (e5m2 is not
+    in the reference, whose backward writes e4m3 bytes whatever the label says)."""
     from linghe_amd.facade.silu import block_silu_impl
 
-    announce("facade BlockSiluFunction", pow2)
+    announce("facade BlockSiluFunction", pow2, gdtype)
     S, B, H = 128, 2, 2048
     g = gen(53)
     x = randn_bf16(g, S, B, H)
@@ -140,7 +150,7 @@ def test_block_silu(gpu, pow2):
     ref = O.silu_and_block_quant_forward(x2, pow2)
     leaf = x.to(gpu).requires_grad_()
     xin = Capture.apply(leaf)
-    out = block_silu_impl(xin, Quantizer(pow2), Quantizer(pow2), FakeQTensor)
+    out = block_silu_impl(xin, Quantizer(pow2), Quantizer(pow2, gtag), FakeQTensor)
     torch.cuda.synchronize()
     assert isinstance(out, FakeQTensor) and tuple(out.shape) == (S, B, H // 2)
     kw = out.kw
@@ -155,8 +165,9 @@ def test_block_silu(gpu, pow2):
     torch.cuda.synchronize()
     gq = Capture.box["grad"]
     assert isinstance(gq, FakeQTensor) and tuple(gq.shape) == (S, B, H)
-    rb = O.silu_and_block_quant_backward(dy.view(S * B, H // 2), x2, pow2)
+    rb = O.silu_and_block_quant_backward(dy.view(S * B, H // 2), x2, pow2, gdtype)
     gk = gq.kw
+    assert gk["fp8_dtype"] is gtag and gk["rowwise_data"].dtype == gdtype and gk["columnwise_data"].dtype == gdtype
     assert tuple(gk["rowwise_data"].shape) == (S, B, H) and tuple(gk["columnwise_data"].shape) == (H, S, B)
     tolb = dict(scale_max_ulp=0, scale_min_within1=1.0) if pow2 else FUSED_BWD
     check_quant_pair("facade.silu.bwd.row", rb[0], rb[1], gk["rowwise_data"].view(S * B, H),
@@ -165,11 +176,11 @@ def test_block_silu(gpu, pow2):
                      gk["columnwise_scale_inv"], **tolb)
 
 
-@pytest.mark.parametrize("is_recomputing", [None, False, True])
-def test_block_batch_weighted_silu(gpu, is_recomputing):
+@pytest.mark.parametrize("is_recomputing,gdtype", [(None, E4M3), (False, E4M3), (True, E4M3), (None, E5M2)])
+def test_block_batch_weighted_silu(gpu, is_recomputing, gdtype):
     from linghe_amd.facade.silu import block_batch_weighted_silu_impl
 
-    announce("facade BlockBatchWeightedSiluFunction", is_recomputing)
+    announce("facade BlockBatchWeightedSiluFunction", is_recomputing, gdtype)
     counts = [160, 0, 96, 272, 16, 128, 33, 64]
     bs, N = sum(counts), 1024
     g = gen(54)
@@ -181,7 +192,8 @@ def test_block_batch_weighted_silu(gpu, is_recomputing):
     wd = w.to(gpu).requires_grad_()
     cnt = torch.tensor(counts, dtype=torch.int32, device=gpu)
     qs = [Quantizer() for _ in counts]
-    out = block_batch_weighted_silu_impl(Capture.apply(leaf), wd, cnt, counts, qs, qs, FakeQTensor,
+    gqs = [Quantizer(dtype=gdtype) for _ in counts]
+    out = block_batch_weighted_silu_impl(Capture.apply(leaf), wd, cnt, counts, qs, gqs, FakeQTensor,
                                          is_recomputing=is_recomputing)
     torch.cuda.synchronize()
     assert isinstance(out, FakeQTensor) and tuple(out.shape) == (bs, N // 2)
@@ -197,8 +209,9 @@ def test_block_batch_weighted_silu(gpu, is_recomputing):
     torch.autograd.backward([out], [dy.to(gpu)])
     torch.cuda.synchronize()
     gq = Capture.box["grad"]
-    rb = O.batch_weighted_silu_and_block_quant_backward(dy, x, w, counts, False)
+    rb = O.batch_weighted_silu_and_block_quant_backward(dy, x, w, counts, False, gdtype)
     assert isinstance(gq, FakeQTensor) and tuple(gq.shape) == (bs, N)
+    assert gq.kw["quantizer"] is gqs and gq.kw["fp8_dtype"] == gdtype and gq.kw["rowwise_data"].dtype == gdtype
     check_quant_pair("facade.batch.bwd.row", rb[0], rb[1], gq.kw["rowwise_data"],
                      gq.kw["rowwise_scale_inv"].view(-1), **FUSED_BWD)
     check_quant_pair("facade.batch.bwd.col", rb[3], rb[4], gq.kw["columnwise_data"].view(-1),
