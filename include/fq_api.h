@@ -110,6 +110,20 @@ int64_t fq_rmsnorm_bwd_num_partials(int64_t M, int64_t n);
 int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx, float* dgamma,
                    float* dgamma_partials, int64_t n_partials, int64_t M, int64_t n, float eps, void* stream);
 
+/* fq_rmsnorm_bwd for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same inputs, outputs and results as
+ * fq_rmsnorm_bwd, but the dgamma partial rows live in a fixed 16 MiB array in
+ * the library's own device memory (one copy per GPU, held until the process
+ * ends) instead of a caller-provided buffer; the call allocates and frees
+ * nothing.  n <= 8192 as for every RMSNorm entry point; anything whose partial
+ * rows would not fit the array is refused with FQ_ERR_SHAPE.  Calls on one GPU
+ * share that GPU's array: calls that may overlap in time (different streams
+ * without ordering) race.  The array's device address is looked up on the first
+ * call on each device. */
+int fq_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
+                           float* dgamma, int64_t M, int64_t n, float eps, void* stream);
+
 /* triton_rms_norm_and_block_quant_forward, linghe/utils/norm.py:343-502.
  * mode 0: writes q, s, rstd.  mode 1: reads rstd, writes qt, st.
  * mode 2: writes q, s, rstd, qt, st; runs as two launches on `stream` - the

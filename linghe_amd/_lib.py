@@ -34,6 +34,7 @@ SIGNATURES = {
     "fq_group_quant": [_P, _P, _P, _L, _L, _I, _I, _P],
     "fq_rmsnorm_fwd": [_P, _P, _P, _P, _L, _L, _F, _I, _P],
     "fq_rmsnorm_bwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _P],
+    "fq_rmsnorm_bwd_noalloc": [_P, _P, _P, _P, _P, _P, _L, _L, _F, _P],
     "fq_rmsnorm_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _I, _I, _P],
     "fq_rmsnorm_router_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _I, _P],
     "fq_swiglu_quant_fwd": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],

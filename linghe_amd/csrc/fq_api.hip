@@ -175,6 +175,26 @@ int fq_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, const float
                       fn);
 }
 
+int fq_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
+                           float* dgamma, int64_t M, int64_t n, float eps, void* stream) {
+  const char* fn = "fq_rmsnorm_bwd_noalloc";
+  int rc = check_norm_shape(fn, M, n);
+  if (rc) return rc;
+  FQ_REQUIRE(dgamma, FQ_ERR_ARG, "%s: dgamma is NULL", fn);
+  const int64_t need = fq::rmsnorm_bwd_partials(M) * n * (int64_t)sizeof(float);
+  FQ_REQUIRE(need <= fq::rmsnorm_bwd_static_scratch_bytes(), FQ_ERR_SHAPE,
+             "%s: %lld bytes of dgamma partials exceed the library's fixed %lld-byte scratch array", fn,
+             (long long)need, (long long)fq::rmsnorm_bwd_static_scratch_bytes());
+  if (M > 0) {
+    FQ_REQUIRE(dy && x && gamma && dx, FQ_ERR_ARG, "%s: NULL pointer", fn);
+    FQ_REQUIRE(aligned16(dy) && aligned16(x) && aligned16(gamma) && aligned16(dx), FQ_ERR_ARG,
+               "%s: misaligned pointer", fn);
+  }
+  return check_launch(fq::launch_rmsnorm_bwd_static(dy, x, gamma, rstd, dx, dgamma, M, (int)n, eps,
+                                                    (hipStream_t)stream),
+                      fn);
+}
+
 int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, float* rstd, void* qt, float* st,
                          int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
                          void* stream) {

@@ -40,6 +40,11 @@ hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, 
                               float* dgamma, float* dg_part, int64_t n_partials, int64_t M, int n, float eps,
                               hipStream_t stream);
 
+// the same with the dgamma partial rows in the library's own fixed device array
+int64_t rmsnorm_bwd_static_scratch_bytes();
+hipError_t launch_rmsnorm_bwd_static(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
+                                     float* dgamma, int64_t M, int n, float eps, hipStream_t stream);
+
 hipError_t launch_group_quant(const void* x, void* q, float* s, int64_t n_groups, int round_scale, int kind,
                               hipStream_t stream);
 

@@ -11,6 +11,8 @@
 // (one 128-bit load each); 16 consecutive lanes therefore share a 128-column
 // quantisation group.  The next row is prefetched while the current one is
 // processed.
+#include <mutex>
+
 #include "fq_device.cuh"
 #include "fq_launch.h"
 
@@ -634,6 +636,55 @@ hipError_t launch_rmsnorm_bwd(const void* dy, const void* x, const void* gamma, 
   hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((n + 63) / 64)), dim3(1024), 0, stream, dg_part, dgamma, (int)P,
                      n);
   return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm backward for callers that cannot allocate: the dgamma partial rows live
+// in a fixed array in device memory instead of a caller-provided buffer.
+// Every GPU the library runs on holds its own copy of the array (16 MiB) at its
+// own address until the process ends; the address is looked up once per device,
+// with that device current, and kernels only ever see the looked-up pointer.
+// The kernels write every partial row they later read, so nothing is cleared
+// between calls; two calls that overlap in time on one GPU share the array and race.
+// ---------------------------------------------------------------------------
+constexpr int64_t kStaticPartialRows = 512;    // the most rmsnorm_bwd_partials() returns
+constexpr int64_t kStaticPartialWidth = 8192;  // the widest row the RMSNorm kernels accept
+static __device__ __align__(256) float scratch[kStaticPartialRows * kStaticPartialWidth];
+
+int64_t rmsnorm_bwd_static_scratch_bytes() { return (int64_t)sizeof(float) * kStaticPartialRows * kStaticPartialWidth; }
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device
+hipError_t static_scratch_ptr(float** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return err;
+    if (p == nullptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = (float*)p;
+  }
+  *out = g_scratch_ptr[dev];
+  return hipSuccess;
+}
+}  // namespace
+
+hipError_t launch_rmsnorm_bwd_static(const void* dy, const void* x, const void* gamma, const float* rstd, void* dx,
+                                     float* dgamma, int64_t M, int n, float eps, hipStream_t stream) {
+  const int64_t P = rmsnorm_bwd_partials(M);
+  if (P > kStaticPartialRows || n > kStaticPartialWidth) return hipErrorInvalidValue;
+  float* part = nullptr;
+  const hipError_t err = static_scratch_ptr(&part);
+  if (err != hipSuccess) return err;
+  return launch_rmsnorm_bwd(dy, x, gamma, rstd, dx, dgamma, part, P, M, n, eps, stream);
 }
 
 hipError_t launch_group_quant(const void* x, void* q, float* s, int64_t n_groups, int round_scale, int kind,
