@@ -76,13 +76,16 @@ def assert_codes(ref, got, name="codes", min_identical=0.9999, max_step=1):
     return rep
 
 
-def assert_scales(ref, got, name="scales", max_ulp=1, min_within_1ulp=1.0, outlier_rel=0.0,
-                  outlier_frac=0.0):
-    """All scales within max_ulp and at least min_within_1ulp of them within
-    1 ulp.  Optionally up to outlier_frac of the scales may exceed max_ulp if
-    their relative difference stays below outlier_rel: the amax of a group of
-    very few elements can be a value that suffered cancellation, whose last
-    bits then carry no information."""
+def assert_scales(ref, got, name="scales", max_ulp=1, min_within_1ulp=1.0, truth=None, bound=None):
+    """All scales within max_ulp of the oracle's and at least min_within_1ulp of them
+    within 1 ulp.
+
+    truth / bound (optional, fp64, same layout as the scales): the real-number value
+    of every scale and the first-order error bound of an fp32 evaluation of it.  With
+    them a scale may be further than max_ulp from the oracle's only where the element
+    that makes the group's amax is ill-conditioned (a cancellation): the group's own
+    bound must exceed max_ulp / 2 ulps, and BOTH sides must lie within that bound of
+    the true value.  Without them nothing may exceed max_ulp."""
     rep = compare_scales(ref, got)
     if rep.total == 0:
         return rep
@@ -90,11 +93,22 @@ def assert_scales(ref, got, name="scales", max_ulp=1, min_within_1ulp=1.0, outli
     frac = rep.within_1ulp / rep.total
     beyond = d > max_ulp
     ok = frac >= min_within_1ulp
+    n_ill = 0
     if bool(beyond.any()):
-        rel = ((ref.float() - got.float()).abs() / ref.float().abs().clamp_min(1e-37))[beyond]
-        ok = ok and float(rel.max()) <= outlier_rel and int(beyond.sum()) <= outlier_frac * rep.total
+        if truth is None:
+            ok = False
+        else:
+            t = truth.reshape(-1)[beyond.reshape(-1)]
+            b = bound.reshape(-1)[beyond.reshape(-1)]
+            ulp = torch.ldexp(torch.ones_like(t), torch.frexp(t.float().double())[1] - 24)
+            ill = b > 0.5 * max_ulp * ulp
+            g = got.detach().float().reshape(-1)[beyond.reshape(-1)].double()
+            r = ref.detach().float().reshape(-1)[beyond.reshape(-1)].double()
+            ok = ok and bool(ill.all()) and bool(((g - t).abs() <= b).all()) and bool(((r - t).abs() <= b).all())
+            n_ill = int(ill.sum())
     assert ok, (f"{name}: exact {rep.exact}/{rep.total}, <=1ulp {rep.within_1ulp}, "
-                f"max {rep.max_ulp} ulp, beyond {max_ulp} ulp: {int(beyond.sum())}")
+                f"max {rep.max_ulp} ulp, beyond {max_ulp} ulp: {int(beyond.sum())} "
+                f"(of which ill-conditioned and within their bound: {n_ill})")
     return rep
 
 

@@ -47,13 +47,14 @@ def zipf_counts(total, n_experts, seed, n_empty=4, s=1.1):
 
 
 def check_quant_pair(name, ref_codes, ref_scales, got_codes, got_scales, *, scale_max_ulp=1,
-                     scale_min_within1=1.0, min_identical=0.9999, max_step=1, outlier_rel=0.0,
-                     outlier_frac=0.0):
+                     scale_min_within1=1.0, min_identical=0.9999, max_step=1, truth=None, bound=None):
+    """truth / bound: fp64 scales and their fp32 error bounds (tests/truth.py), in the
+    layout of got_scales; see oracle.compare.assert_scales."""
     got_codes = got_codes.detach().cpu()
     got_scales = got_scales.detach().cpu()
     srep = C.assert_scales(ref_scales.reshape(-1), got_scales.reshape(-1), name + ".scale",
                            max_ulp=scale_max_ulp, min_within_1ulp=scale_min_within1,
-                           outlier_rel=outlier_rel, outlier_frac=outlier_frac)
+                           truth=truth, bound=bound)
     crep = C.assert_codes(ref_codes.reshape(-1), got_codes.reshape(-1), name + ".codes",
                           min_identical=min_identical, max_step=max_step)
     print(f"[parity] {name}: codes identical {crep.identical}/{crep.total} max_step {crep.max_step}; "

@@ -159,10 +159,10 @@ def test_cfg5_rmsnorm_large_full(gpu):
     _, _, _, qt1, st1 = fwd(xd, wd, eps, rms=r, output_mode=1)
     torch.cuda.synchronize()
     ref = O.rms_norm_and_block_quant_forward(x, w, eps)
-    # 7168 heavy-tailed terms per row: torch's CPU sum and the kernel's sum are each
-    # about one ulp from the exact sum of squares, and 1/sqrt(ss/n + eps) turns a
-    # 2-ulp difference of ss into up to 2 ulps of the statistic in ~10 % of the rows
-    tol = dict(FUSED_NORM, scale_min_within1=0.85)
+    # 7168 heavy-tailed terms per row: torch's CPU sum is about one ulp from the exact
+    # sum of squares (the kernel's is the exact sum rounded once), and 1/sqrt(ss/n + eps)
+    # turns that into up to 2 ulps of the statistic in ~7 % of the rows
+    tol = dict(FUSED_NORM)
     check_quant_pair("cfg5b.row", ref[0], ref[1], q, s, **tol)
     check_quant_pair("cfg5b.col", ref[3], ref[4], qt, st, **tol)
     C.assert_scales(ref[2], r.cpu(), "cfg5.rstd", max_ulp=4, min_within_1ulp=0.9)

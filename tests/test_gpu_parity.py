@@ -6,21 +6,23 @@ compared with the CPU oracle on identical seeded inputs.
 Acceptance (stricter than the reference's output_check):
   * FP8 codes: >= 99.99 % bit-identical, every mismatch exactly one code step;
   * fp32 scales of the plain quantisers: bit-identical;
-  * fp32 scales of the fused ops: the value whose amax makes the scale is itself
-    the result of fp32 arithmetic whose last bits depend on the reduction order
-    of sum(x^2) (RMSNorm) or on the exp implementation (SwiGLU), and dividing by
-    448 can turn a 1-ulp difference of amax into 2 ulps of scale (the quotient's
-    mantissa is 8/7 of the dividend's).
-      - SwiGLU family: >= 95 % within 1 ulp (94 % in the backward), none beyond
-        8 ulp (a chain of six roundings after an exp that is itself good to
-        1-2 ulp on either side), except that in the backward at most 0.5 % of
-        the scales may differ by up to 1e-4 relative: dx1 = h*s + h*x1*(1-s)*s
-        cancels for x1 near -1.28, and the amax of a group of one or two rows
-        (ragged experts) can be such an element;
-      - RMSNorm family against the pure oracle: >= 90 % within 1 ulp, none
-        beyond 8 ulp (the statistic itself differs by up to 2 ulp from torch's
-        CPU sum for heavy-tailed rows); against the oracle evaluated with the
-        kernel's own statistic: bit-identical scales and codes;
+  * fp32 scales of the fused ops: oracle and kernel are two fp32 evaluations of the
+    same expression, each up to 3-5 ulp from the real-number value (measured
+    against fp64 in tests/test_gpu_truth.py: the kernel is as close to it as the
+    oracle, closer after an RMSNorm), so they differ from EACH OTHER by up to 6 ulp.
+    The limits below are the largest differences measured over every shape here
+    and the benchmark configurations:
+      - SwiGLU forward: none beyond 5 ulp, >= 98 % within 1 ulp (torch's CPU sigmoid
+        is 1/(1+exp(-x)) with a vectorised 2-ulp exp, the kernel's a hardware exp2);
+      - SwiGLU backward: none beyond 6 ulp, >= 98 % within 1 ulp, except where
+        dx1 = h*s + h*x1*(1-s)*s cancels (x1 near -1.28) in the element that makes a
+        group's amax - a group of one or two rows of a ragged expert: there both
+        sides must lie within that element's own error bound of the fp64 value;
+      - RMSNorm family against the pure oracle: none beyond 6 ulp, >= 90 % within
+        1 ulp (torch's CPU sum of squares is itself about one ulp from the exact
+        sum, and 1/sqrt turns that into 1-2 ulp of the statistic); against the
+        oracle evaluated with the kernel's own statistic: bit-identical scales and
+        codes;
   * bf16 outputs: >= 99.5 % identical, the rest within 2 bf16 ulps or, where
     dx = r*g*w - coef*x cancels, within 2^-9 of the tensor's largest magnitude.
 """
@@ -29,14 +31,15 @@ import torch
 
 from oracle import compare as C
 from oracle import fq_oracle as O
+from tests import truth as T
 from tests.helpers import (E4M3, E5M2, announce, check_quant_pair, gamma_bf16, gen, randn_bf16,
                            zipf_counts)
 
 pytestmark = pytest.mark.gpu
 
-FUSED = dict(scale_max_ulp=6, scale_min_within1=0.97)                      # SwiGLU forward
-FUSED_BWD = dict(scale_max_ulp=6, scale_min_within1=0.97, outlier_rel=1e-4, outlier_frac=0.005)
-FUSED_NORM = dict(scale_max_ulp=8, scale_min_within1=0.9)                   # RMSNorm vs pure oracle
+FUSED = dict(scale_max_ulp=5, scale_min_within1=0.98)        # SwiGLU forward
+FUSED_BWD = dict(scale_max_ulp=6, scale_min_within1=0.98)    # SwiGLU backward (+ the conditioned escape, see above)
+FUSED_NORM = dict(scale_max_ulp=6, scale_min_within1=0.9)    # RMSNorm vs pure oracle
 EXACT = dict(scale_max_ulp=0, scale_min_within1=1.0, min_identical=1.0)
 
 
@@ -268,8 +271,10 @@ def test_silu_and_block_quant_bwd(gpu, M, N, coef, gcoef, dtype):
     torch.cuda.synchronize()
     assert dq.shape == (M, N) and ds.shape == (N // 128, M) and dqt.shape == (N, M) and dst.shape == (M // 128, N)
     assert dq.dtype == dtype
-    check_quant_pair("silu.bwd.row", ref[0], ref[1], dq, ds, **FUSED_BWD)
-    check_quant_pair("silu.bwd.col", ref[2], ref[3], dqt, dst, **FUSED_BWD)
+    v, err, _ = T.swiglu_grad_values(dy, x)
+    sr, br, sc, bc = T.scale_bounds(v, err, O.fp8_max(dtype))
+    check_quant_pair("silu.bwd.row", ref[0], ref[1], dq, ds, truth=sr, bound=br, **FUSED_BWD)
+    check_quant_pair("silu.bwd.col", ref[2], ref[3], dqt, dst, truth=sc, bound=bc, **FUSED_BWD)
 
 
 def _batched_case(gpu, counts, N, coef, gcoef, seed, wdtype=torch.float32):
@@ -302,8 +307,10 @@ def _batched_case(gpu, counts, N, coef, gcoef, seed, wdtype=torch.float32):
     assert dq.shape == (bs, N) and dw.shape == w.shape and dw.dtype == w.dtype
     if bs == 0:
         return
-    check_quant_pair("batch.bwd.row", rb[0], rb[1], dq, ds.view(-1), **FUSED_BWD)
-    check_quant_pair("batch.bwd.col", rb[3], rb[4], dqt.view(-1), dst.view(-1), **FUSED_BWD)
+    v, err, _ = T.swiglu_grad_values(dy, x, w.float())
+    sr, br, sc, bc = T.scale_bounds_per_expert(v, err, counts)
+    check_quant_pair("batch.bwd.row", rb[0], rb[1], dq, ds.view(-1), truth=sr, bound=br, **FUSED_BWD)
+    check_quant_pair("batch.bwd.col", rb[3], rb[4], dqt.view(-1), dst.view(-1), truth=sc, bound=bc, **FUSED_BWD)
     tol = 2e-2 if wdtype == torch.bfloat16 else 1e-4
     torch.testing.assert_close(dw.cpu().float(), rb[2].float(), rtol=tol,
                                atol=tol * max(float(rb[2].abs().max()), 1e-30))
