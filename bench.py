@@ -1,14 +1,21 @@
 #!/usr/bin/env python3
 """Benchmark of the fused blockwise-FP8 quantisation path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs all|cfg1,cfg2,...] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--configs all|cfg1,cfg2,...] [--no-cpu]
 
 A "step" is one call of the entry point of a configuration on one batch of
 synthetic (seeded) input that is already resident in HBM.  Calls go through
 the C ABI with preallocated outputs; K steps are timed between two events on
-the launch stream.  Buffers rotate over enough copies to exceed twice the
+the launch stream, R times over, and the median loop is reported (with the
+fastest and slowest).  Buffers rotate over enough copies to exceed twice the
 256 MB Infinity Cache, so the figure is an HBM figure ("cold"); the same loop
 on one fixed set of buffers gives the cache-resident ("hot") figure.
+
+Beside each configuration: the time a kernel that does no work needs to read
+and write the configuration's algorithmic byte counts (`stream_us`, the
+measured ceiling of this device for those bytes), the HBM traffic per call
+measured with the profiler's counters (from profiles/hbm_traffic_per_config.md)
+and the torch CPU oracle timed on the host cores.
 
 Prints ONE JSON line: the headline metric is us/call of RMSNorm + 1x128 quant
 forward on bf16 [8192, 2048] (output_mode 2); the other configurations are
@@ -40,9 +47,10 @@ def _p(t):
 class Case:
     """One configuration: `sets` buffer sets and a launcher taking a set index."""
 
-    def __init__(self, name, entry, shape, algo_bytes, make_set, launch, cpu_fn):
+    def __init__(self, name, entry, shape, rw_bytes, make_set, launch, cpu_fn):
         self.name, self.entry, self.shape = name, entry, shape
-        self.algo_bytes = algo_bytes
+        self.read_bytes, self.write_bytes = rw_bytes          # algorithmic bytes read / written per call
+        self.algo_bytes = self.read_bytes + self.write_bytes
         self.make_set, self.launch, self.cpu_fn = make_set, launch, cpu_fn
         self.sets = []
 
@@ -99,7 +107,7 @@ def build_cases(names, dev):
         if mode == 2:
             label += " two passes"
         return Case(name, label, [M, n],
-                    configs.bytes_rmsnorm_quant(M, n, mode), make_set, launch, cpu_fn)
+                    configs.rw_rmsnorm_quant(M, n, mode), make_set, launch, cpu_fn)
 
     lazy = {}
 
@@ -135,7 +143,7 @@ def build_cases(names, dev):
             return O.silu_and_block_quant_forward(x_cpu, False)
 
         return Case("cfg2", "triton_silu_and_block_quant_forward(output_mode=2)", [M, N],
-                    configs.bytes_swiglu_fwd(M, n), make_set, launch, cpu_fn)
+                    configs.rw_swiglu_fwd(M, n), make_set, launch, cpu_fn)
 
     add("cfg2", build=swiglu_fwd_case)
 
@@ -173,7 +181,7 @@ def build_cases(names, dev):
             def cpu_fn():
                 from oracle import fq_oracle as O
                 return O.batch_weighted_silu_and_block_quant_backward(dy_cpu, x_cpu, w_cpu, counts, False)
-            nbytes = configs.bytes_batched_swiglu_bwd(M, n, counts)
+            nbytes = configs.rw_batched_swiglu_bwd(M, n, counts)
             entry = "triton_batch_weighted_silu_and_block_quant_backward"
         else:
             def launch(s):
@@ -182,7 +190,7 @@ def build_cases(names, dev):
             def cpu_fn():
                 from oracle import fq_oracle as O
                 return O.batch_weighted_silu_and_block_quant_forward(x_cpu, w_cpu, counts, False)
-            nbytes = configs.bytes_batched_swiglu_fwd(M, n, counts)
+            nbytes = configs.rw_batched_swiglu_fwd(M, n, counts)
             entry = "triton_batch_weighted_silu_and_block_quant_forward(output_mode=2)"
         c = Case("cfg3b" if backward else "cfg3", entry, [M, N], nbytes, make_set, launch, cpu_fn)
         c.extra = dict(n_experts=E, blocks=blocks, empty_experts=sum(1 for v in counts if v == 0),
@@ -217,7 +225,7 @@ def build_cases(names, dev):
             return O.silu_and_block_quant_backward(dy_cpu, x_cpu, False, dt)
 
         return Case(name, "triton_silu_and_block_quant_backward(fp8=%s)" % str(dt).split(".")[-1], [M, N],
-                    configs.bytes_swiglu_bwd(M, n), make_set, launch, cpu_fn)
+                    configs.rw_swiglu_bwd(M, n), make_set, launch, cpu_fn)
 
     add("cfg4", build=lambda: swiglu_bwd_case(_lib.FQ_E4M3, "cfg4"))
     add("cfg4_e5m2", build=lambda: swiglu_bwd_case(_lib.FQ_E5M2, "cfg4_e5m2"))
@@ -245,7 +253,7 @@ def build_cases(names, dev):
             from oracle import fq_oracle as O
             return O.rms_norm_backward(x_cpu, g_cpu, dy_cpu, eps)
 
-        return Case("cfg5a", "triton_rms_norm_backward", [M, n], configs.bytes_rmsnorm_bwd(M, n), make_set, launch,
+        return Case("cfg5a", "triton_rms_norm_backward", [M, n], configs.rw_rmsnorm_bwd(M, n), make_set, launch,
                     cpu_fn)
 
     add("cfg5a", build=rms_bwd_case)
@@ -279,7 +287,7 @@ def build_cases(names, dev):
             return O.batch_block_pad_permute_with_indices(x_cpu, d["indices_unpadded"], probs_cpu, counts, False)
 
         return Case("next_permute", "triton_batch_block_pad_permute_with_indices", [M, N],
-                    configs.bytes_permute_pad_quant(N, counts), make_set, launch, cpu_fn)
+                    configs.rw_permute_pad_quant(N, counts), make_set, launch, cpu_fn)
 
     add("next_permute", build=permute_case)
 
@@ -309,7 +317,7 @@ def build_cases(names, dev):
             from oracle import fq_oracle as O
             return O.weighted_silu_backward(dy_cpu, x_cpu, w_cpu) if backward else O.weighted_silu_forward(x_cpu, w_cpu)
 
-        nbytes = (2 * M * N + 2 * M * (N // 2) + 4 * M) + ((2 * M * N + 4 * M) if backward else 0)
+        nbytes = configs.rw_weighted_silu(M, N // 2, backward)
         return Case("next_wsilu_bwd" if backward else "next_wsilu_fwd",
                     "triton_weighted_silu_backward" if backward else "triton_weighted_silu_forward", [M, N], nbytes,
                     make_set, launch, cpu_fn)
@@ -336,7 +344,7 @@ def build_cases(names, dev):
             return O.block_quant_128(x_cpu, True)
 
         return Case("next_block_quant", "triton_block_quant(round_scale=True)", [M, N],
-                    3 * M * N + 4 * (M // 128) * (N // 128), make_set, launch, cpu_fn)
+                    configs.rw_block_quant(M, N), make_set, launch, cpu_fn)
 
     add("next_block_quant", build=block_quant_case)
 
@@ -368,46 +376,58 @@ def build_cases(names, dev):
             return O.rms_gemm_block_quant_forward(x_cpu, nw_cpu, rw_cpu)
 
         c = Case("next_router", "triton_rms_norm_fp32_gemm_block_quant_forward(output_mode=0)", [M, N, K],
-                 5 * M * K + 4 * M * N + 4 * (K // 128) * M + 4 * M + 2 * N * K + 2 * K, make_set, launch, cpu_fn)
+                 configs.rw_router(M, N, K), make_set, launch, cpu_fn)
         c.extra = {"gemm_flops": 2 * M * N * K}
         return c
 
     add("next_router", build=router_case)
 
-    # ---------------------------------------------------------------- plain copy of known size
-    # (calibration of the FETCH_SIZE / WRITE_SIZE counters: reads and writes 256 MiB)
-    def copy_case():
-        nbytes = 256 << 20
+    # ---------------------------------------------------------------- the no-work stream kernel on a known size
+    # (the read / copy rates of the memory system, and the calibration of FETCH_SIZE / WRITE_SIZE)
+    def stream_case(name, read_mib, write_mib):
+        rb, wb = read_mib << 20, write_mib << 20
+        sink = torch.zeros(16, device=dev, dtype=torch.uint8)
 
         def make_set():
-            return dict(src=torch.zeros(nbytes // 2, device=dev, dtype=torch.bfloat16),
-                        dst=torch.empty(nbytes // 2, device=dev, dtype=torch.bfloat16))
+            s = dict(src=torch.zeros(max(rb, 16), device=dev, dtype=torch.uint8),
+                     dst=torch.empty(max(wb, 16), device=dev, dtype=torch.uint8))
+            s["args"] = (_p(s["src"]), rb, _p(s["dst"]), wb, _p(sink), 0, stream)
+            return s
 
         def launch(s):
-            s["dst"].copy_(s["src"])
+            _lib.check(L.fq_stream_rw(*s["args"]))
 
-        return Case("copy", "torch copy_ of 256 MiB (counter calibration)", [nbytes], 2 * nbytes, make_set, launch,
-                    lambda: None)
+        return Case(name, "fq_stream_rw: read %d MiB, write %d MiB, no arithmetic" % (read_mib, write_mib),
+                    [rb, wb], (rb, wb), make_set, launch, None)
 
-    add("copy", build=copy_case)
+    add("stream_read", build=lambda: stream_case("stream_read", 256, 0))
+    add("stream_copy", build=lambda: stream_case("stream_copy", 256, 256))
     return cases
 
 
-def time_loop(case, sets, steps, warmup):
-    """us per call: `steps` back-to-back launches between two events on the
-    launch stream (the current torch stream), rotating over `sets`."""
+def time_loop(launch, sets, steps, warmup, repeats):
+    """us per call, one figure per repeat: `steps` back-to-back launches between two
+    events on the launch stream (the current torch stream), rotating over `sets`."""
     k = len(sets)
     for i in range(warmup):
-        case.launch(sets[i % k])
-    torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for i in range(steps):
-        case.launch(sets[i % k])
-    end.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(end) * 1000.0 / steps
+        launch(sets[i % k])
+    out = []
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(steps):
+            launch(sets[i % k])
+        end.record()
+        torch.cuda.synchronize()
+        out.append(start.elapsed_time(end) * 1000.0 / steps)
+    return sorted(out)
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2] if len(xs) % 2 else 0.5 * (xs[len(xs) // 2 - 1] + xs[len(xs) // 2])
 
 
 def time_single_calls(case, sets, calls, warmup):
@@ -432,42 +452,68 @@ def time_single_calls(case, sets, calls, warmup):
     return t[len(t) // 2], sum(kept) / len(kept)
 
 
-def time_cpu(case, budget_s):
-    """oracle on the host cores: 1 warm-up, then min over up to 20 runs within the budget."""
-    t0 = time.perf_counter()
+def time_cpu(case):
+    """the oracle on the host cores: 1 warm-up, then the minimum of 3 runs (us)."""
     case.cpu_fn()
-    first = time.perf_counter() - t0
-    runs = [first]
-    spent = first
-    while len(runs) < 21 and spent + runs[-1] < budget_s:
+    runs = []
+    for _ in range(3):
         t0 = time.perf_counter()
         case.cpu_fn()
         runs.append(time.perf_counter() - t0)
-        spent += runs[-1]
-    best = min(runs[1:]) if len(runs) > 1 else runs[0]
-    return best * 1e6, len(runs)
+    return min(runs) * 1e6
 
 
-# HBM bytes per call of the headline entry point (statistic kernel + tile kernel),
-# from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
-# counters read for the 256 MiB `copy` case (x2.0 and x1.0):
-# fetched 33.63 + 33.99 MB, written 0.26 + 34.60 MB; algorithmic bytes are 68.19 MB,
-# the difference is the second read of x.
-CFG1_MEASURED_TRAFFIC_BYTES = 102.48e6
+def stream_ceiling(case, dev, stream, steps, warmup, repeats):
+    """us for the no-work kernel to read and write this configuration's algorithmic byte
+    counts, cold buffers: what the memory system alone takes for the same bytes.  The
+    better of plain and non-temporal accesses."""
+    from linghe_amd import _lib
+    rb, wb = (case.read_bytes + 15) // 16 * 16, (case.write_bytes + 15) // 16 * 16
+    n_sets = max(2, min(16, (2 * INFINITY_CACHE_BYTES + (64 << 20)) // max(1, rb + wb) + 1))
+    sink = torch.zeros(16, device=dev, dtype=torch.uint8)
+    sets = [(torch.zeros(max(rb, 16), device=dev, dtype=torch.uint8),
+             torch.empty(max(wb, 16), device=dev, dtype=torch.uint8)) for _ in range(n_sets)]
+    best = None
+    for nt in (0, 1):
+        def launch(s, nt=nt):
+            _lib.check(_lib.lib.fq_stream_rw(s[0].data_ptr(), rb, s[1].data_ptr(), wb, sink.data_ptr(), nt, stream))
+        t = median(time_loop(launch, sets, steps, warmup, repeats))
+        best = t if best is None else min(best, t)
+    return best
+
+
+def load_traffic_table():
+    """Measured HBM bytes per call and configuration, from the tracked profiler summary
+    (rows `| config | fetched MB | written MB | total MB |`): the digits printed here are
+    the digits of that file.  Absent file or row -> None."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_per_config.md")
+    table = {}
+    if os.path.exists(path):
+        for line in open(path):
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            if len(cells) >= 4:
+                try:
+                    table[cells[0]] = dict(fetched=float(cells[1]) * 1e6, written=float(cells[2]) * 1e6,
+                                           total=float(cells[3]) * 1e6)
+                except ValueError:
+                    pass
+    return table
+
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
-       "next_permute",
-       "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router"]
+       "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router",
+       "stream_read", "stream_copy"]
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=7, help="timed loops of --steps calls per figure; the median is reported")
     ap.add_argument("--configs", default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
-    ap.add_argument("--cpu-all", action="store_true", help="time the CPU oracle for every config, not only cfg1")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the no-work stream kernel on each config's bytes")
     ap.add_argument("--no-headline", action="store_true",
                     help="profiling aid: run only the named configs and print their results without the headline line")
     ap.add_argument("--hot-only", action="store_true", help="profiling aid: one buffer set, no rotation")
@@ -484,35 +530,51 @@ def main():
         names = ["cfg1"] + names
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
     builders = build_cases(set(names), dev)
+    traffic = load_traffic_table()
     results = {}
-    headline_cpu = None
     for name in names:
         case = builders[name]["build"]()
         case.allocate()
         if args.hot_only:
             case.sets = case.sets[:1]
-        cold = time_loop(case, case.sets, args.steps, args.warmup)
-        hot = cold if args.hot_only else time_loop(case, case.sets[:1], args.steps, args.warmup)
+        cold = time_loop(case.launch, case.sets, args.steps, args.warmup, args.repeats)
+        hot = cold if args.hot_only else time_loop(case.launch, case.sets[:1], args.steps, args.warmup,
+                                                   min(3, args.repeats))
         med, trimmed = time_single_calls(case, case.sets, max(10, min(args.steps, 200)), min(args.warmup, 10))
-        gbs = case.algo_bytes / cold / 1e3
+        us = median(cold)
+        gbs = case.algo_bytes / us / 1e3
         r = dict(entry=case.entry, shape=case.shape, algorithmic_bytes=case.algo_bytes,
-                 us_per_call=round(cold, 3), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
-                 us_per_call_hot=round(hot, 3), gb_per_s_hot=round(case.algo_bytes / hot / 1e3, 1),
+                 algorithmic_bytes_read=case.read_bytes, algorithmic_bytes_written=case.write_bytes,
+                 us_per_call=round(us, 3), us_per_call_min=round(cold[0], 3), us_per_call_max=round(cold[-1], 3),
+                 timed_loops=len(cold), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
+                 us_per_call_hot=round(median(hot), 3), gb_per_s_hot=round(case.algo_bytes / median(hot) / 1e3, 1),
                  us_single_call_median=round(med, 3), us_single_call_trimmed_mean=round(trimmed, 3),
                  buffer_sets=len(case.sets))
         if hasattr(case, "extra"):
             r.update(case.extra)
-        if not args.no_cpu and (name == "cfg1" or args.cpu_all):
-            cpu_us, n_runs = time_cpu(case, budget_s=20.0)
-            r["cpu_us_per_call"] = round(cpu_us, 1)
-            r["cpu_runs"] = n_runs
-            if name == "cfg1":
-                headline_cpu = (cpu_us, n_runs)
-        results[name] = r
-        print(f"[bench] {name}: {cold:.2f} us cold ({gbs:.0f} GB/s, {100 * gbs / HBM_PEAK_GBS:.1f}% of peak), "
-              f"{hot:.2f} us hot", file=sys.stderr, flush=True)
+        # the buffers of the case are released before the ceiling and the CPU leg allocate theirs
         case.sets = []
+        torch.cuda.empty_cache()
+        if not args.no_ceiling and not name.startswith("stream_"):
+            ceil_us = stream_ceiling(case, dev, stream, args.steps, args.warmup, min(3, args.repeats))
+            r["stream_us"] = round(ceil_us, 3)
+            r["stream_gb_per_s"] = round(case.algo_bytes / ceil_us / 1e3, 1)
+            r["frac_of_stream"] = round(ceil_us / us, 4)
+            torch.cuda.empty_cache()
+        if name in traffic:
+            r["hbm_traffic_bytes"] = traffic[name]["total"]
+            r["hbm_fetched_bytes"] = traffic[name]["fetched"]
+            r["hbm_written_bytes"] = traffic[name]["written"]
+        if not args.no_cpu and case.cpu_fn is not None:
+            r["cpu_us_per_call"] = round(time_cpu(case), 1)
+            r["cpu_threads"] = torch.get_num_threads()
+        results[name] = r
+        print(f"[bench] {name}: {us:.2f} us cold [{cold[0]:.2f} .. {cold[-1]:.2f}] ({gbs:.0f} GB/s, "
+              f"{100 * gbs / HBM_PEAK_GBS:.1f}% of peak"
+              + (f", {100 * r['frac_of_stream']:.0f}% of the no-work kernel's rate" if "stream_us" in r else "")
+              + f"), {median(hot):.2f} us hot", file=sys.stderr, flush=True)
         del case
         torch.cuda.empty_cache()
 
@@ -520,6 +582,12 @@ def main():
         print(json.dumps({"configs": results}))
         return
     head = results["cfg1"]
+    roofline = {"bound": "hbm", "achieved": head["gb_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": head["frac_of_hbm_peak"], "traffic": head.get("hbm_traffic_bytes")}
+    if "stream_us" in head:
+        # what a kernel that only moves cfg1's bytes reaches on this device, and cfg1 against it
+        roofline["copy_ceiling"] = head["stream_gb_per_s"]
+        roofline["frac_of_copy_ceiling"] = head["frac_of_stream"]
     line = {
         "metric": "us/call and achieved HBM GB/s (% of peak), RMSNorm+quant fwd 8192x2048",
         "value": head["us_per_call"],
@@ -531,20 +599,22 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "cfg1: RMSNorm + 1x128/128x1 e4m3 blockwise quant forward, x bf16 [8192,2048], "
-                               "output_mode 2, round_scale False, buffers rotated beyond the Infinity Cache",
+                               "output_mode 2, round_scale False, buffers rotated beyond the Infinity Cache; "
+                               "bf16 in, fp32 arithmetic, fp8 + fp32 scales out; value = median of %d loops of "
+                               "%d calls" % (head["timed_loops"], args.steps),
                    "entry": head["entry"]},
-        "roofline": {"bound": "hbm", "achieved": head["gb_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["frac_of_hbm_peak"], "traffic": CFG1_MEASURED_TRAFFIC_BYTES},
+        "roofline": roofline,
         "configs": results,
     }
-    if headline_cpu is not None:
-        line["cpu_baseline"] = {"value": round(headline_cpu[0], 1), "unit": "us/call",
-                                "cores": torch.get_num_threads(), "kind": "port",
-                                "sample": "cfg1 at full size, torch CPU oracle, 1 warm-up + min of %d calls; "
-                                          "os.cpu_count()=%d" % (max(1, headline_cpu[1] - 1), os.cpu_count())}
+    if "cpu_us_per_call" in head:
+        line["cpu_baseline"] = {"value": head["cpu_us_per_call"], "unit": "us/call",
+                                "cores": head["cpu_threads"], "kind": "port",
+                                "sample": "cfg1 at full size, torch CPU oracle, 1 warm-up + min of 3 calls; "
+                                          "os.cpu_count()=%d; every other config has its own cpu_us_per_call"
+                                          % os.cpu_count()}
     print(json.dumps(line))
 
 

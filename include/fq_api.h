@@ -49,6 +49,17 @@ int fq_version(void);
 /* message of this thread's last failing call ("" if none) */
 const char* fq_last_error(void);
 
+/* Measurement aid with no counterpart in the reference: a kernel that reads
+ * read_bytes from src and writes write_bytes to dst (multiples of 16; the two
+ * need not be equal, either may be 0) with the 16-byte accesses of the product
+ * kernels and no arithmetic.  sink: 16 bytes of device memory that are never
+ * written in practice (they keep the loads alive).  nontemporal != 0 puts the
+ * streaming hint on loads and stores.  bench.py times it on each
+ * configuration's own byte counts (the measured ceiling) and the profiler
+ * counters are calibrated on it. */
+int fq_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink, int nontemporal,
+                 void* stream);
+
 /* triton_blockwise_quant, linghe/quant/block.py:129-170.
  * x bf16 [M,N], N % 128 == 0.  q [M,N], s [N/128, M], qt [N, M], st [ceil(M/128), N]. */
 int fq_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t N,

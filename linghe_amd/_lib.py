@@ -12,7 +12,8 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libfq_gfx950.so"
-LIB_PATH = os.path.join(_HERE, LIB_NAME)
+# LINGHE_FQ_LIB names another build of the same library (same ABI), e.g. one compiled with other tuning macros
+LIB_PATH = os.environ.get("LINGHE_FQ_LIB") or os.path.join(_HERE, LIB_NAME)
 
 FQ_E4M3 = 0
 FQ_E5M2 = 1
@@ -25,6 +26,7 @@ _F = ctypes.c_float
 
 # name -> argtypes, exactly the declarations of include/fq_api.h
 SIGNATURES = {
+    "fq_stream_rw": [_P, _L, _P, _L, _P, _I, _P],
     "fq_blockwise_quant": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_blockwise_quant": [_P, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_pad_permute_quant": [_P, _P, _I, _I, _L, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _P],

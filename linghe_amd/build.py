@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libfq_gfx950.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["fq_api.hip", "fq_tile_kernels.hip", "fq_row_kernels.hip", "fq_router.hip"]
+SOURCES = ["fq_api.hip", "fq_tile_kernels.hip", "fq_row_kernels.hip", "fq_router.hip", "fq_stream.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -53,25 +53,26 @@ def _run(cmd):
         sys.stderr.write(err + "\n")
 
 
-def build_library(extra_flags=(), verbose: bool = False) -> str:
+def build_library(extra_flags=(), verbose: bool = False, csrc: str = CSRC, out: str = LIB_PATH) -> str:
+    """Compile the translation units under `csrc` and link them into `out`."""
     hipcc = _hipcc()
-    objdir = os.path.join(HERE, "build")
+    objdir = os.path.join(os.path.dirname(os.path.abspath(out)), "build")
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
 
     def compile_one(pair):
         src, obj = pair
-        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(csrc, src), "-o", obj]
         if verbose:
             print(" ".join(cmd))
         _run(cmd)
 
     with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
         list(pool.map(compile_one, zip(SOURCES, objs)))
-    tmp = LIB_PATH + ".tmp"
+    tmp = out + ".tmp"
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, out)
+    return out
 
 
 if __name__ == "__main__":

@@ -106,45 +106,90 @@ def next_permute_pad_quant(tokens: int = 16384, n: int = 2048, n_experts: int = 
     return dict(x=x, probs=probs, counts=counts, indices=torch.cat(parts), indices_unpadded=torch.cat(plain))
 
 
-# algorithmic HBM bytes per call (each input read once, each output written once)
-def bytes_rmsnorm_quant(M, n, mode=2):
-    x = 2 * M * n
+# algorithmic HBM bytes per call as (bytes read, bytes written): each input read once, each
+# output written once; scratch (dgamma / dw partial sums, the re-ordered router weight) is
+# not counted
+def rw_rmsnorm_quant(M, n, mode=2):
+    x = 2 * M * n + 2 * n
     row = M * n + 4 * (n // 128) * M
     col = M * n + 4 * ((M + 127) // 128) * n
     if mode == 0:
-        return x + 2 * n + row + 4 * M
+        return x, row + 4 * M
     if mode == 1:
-        return x + 2 * n + 4 * M + col
-    return x + 2 * n + row + col + 4 * M
+        return x + 4 * M, col
+    return x, row + col + 4 * M
 
 
-def bytes_swiglu_fwd(M, n):
-    return 2 * M * 2 * n + 2 * M * n + 4 * (n // 128) * M + 4 * ((M + 127) // 128) * n
+def rw_swiglu_fwd(M, n):
+    return 2 * M * 2 * n, 2 * M * n + 4 * (n // 128) * M + 4 * ((M + 127) // 128) * n
 
 
-def bytes_swiglu_bwd(M, n):
+def rw_swiglu_bwd(M, n):
     N = 2 * n
-    return 2 * M * n + 2 * M * N + 2 * M * N + 4 * (N // 128) * M + 4 * ((M + 127) // 128) * N
+    return 2 * M * n + 2 * M * N, 2 * M * N + 4 * (N // 128) * M + 4 * ((M + 127) // 128) * N
 
 
-def bytes_batched_swiglu_fwd(M, n, counts):
+def rw_batched_swiglu_fwd(M, n, counts):
     blocks = sum((c + 127) // 128 for c in counts)
-    return 2 * M * 2 * n + 4 * M + 2 * M * n + 4 * M * (n // 128) + 4 * blocks * n
+    return 2 * M * 2 * n + 4 * M, 2 * M * n + 4 * M * (n // 128) + 4 * blocks * n
 
 
-def bytes_batched_swiglu_bwd(M, n, counts):
+def rw_batched_swiglu_bwd(M, n, counts):
     blocks = sum((c + 127) // 128 for c in counts)
     N = 2 * n
-    return 2 * M * n + 2 * M * N + 4 * M + 2 * M * N + 4 * M * (N // 128) + 4 * blocks * N + 4 * M
+    return 2 * M * n + 2 * M * N + 4 * M, 2 * M * N + 4 * M * (N // 128) + 4 * blocks * N + 4 * M
 
 
-def bytes_rmsnorm_bwd(M, n):
-    return 2 * (2 * M * n) + 2 * M * n + 2 * n + 4 * n
+def rw_rmsnorm_bwd(M, n):
+    return 2 * (2 * M * n) + 2 * n, 2 * M * n + 4 * n
 
 
-def bytes_permute_pad_quant(n, counts):
+def rw_permute_pad_quant(n, counts):
     """each routed row read once (2 B/element) with its index and prob, both code layouts and scales written"""
     routed = sum(counts)
     padded = sum((c + 15) // 16 * 16 for c in counts)
     blocks = sum((c + 127) // 128 for c in counts)
-    return 2 * routed * n + 4 * padded + 4 * routed + 2 * padded * n + 4 * padded * (n // 128) + 4 * blocks * n + 4 * padded
+    return (2 * routed * n + 4 * padded + 4 * routed,
+            2 * padded * n + 4 * padded * (n // 128) + 4 * blocks * n + 4 * padded)
+
+
+def rw_weighted_silu(M, n, backward):
+    if backward:
+        return 2 * M * 2 * n + 2 * M * n + 4 * M, 2 * M * 2 * n + 4 * M
+    return 2 * M * 2 * n + 4 * M, 2 * M * n
+
+
+def rw_block_quant(M, N):
+    return 2 * M * N, M * N + 4 * (M // 128) * (N // 128)
+
+
+def rw_router(M, N, K):
+    return 2 * M * K + 2 * N * K + 2 * K, 2 * M * K + M * K + 4 * M * N + 4 * (K // 128) * M + 4 * M
+
+
+def bytes_rmsnorm_quant(M, n, mode=2):
+    return sum(rw_rmsnorm_quant(M, n, mode))
+
+
+def bytes_swiglu_fwd(M, n):
+    return sum(rw_swiglu_fwd(M, n))
+
+
+def bytes_swiglu_bwd(M, n):
+    return sum(rw_swiglu_bwd(M, n))
+
+
+def bytes_batched_swiglu_fwd(M, n, counts):
+    return sum(rw_batched_swiglu_fwd(M, n, counts))
+
+
+def bytes_batched_swiglu_bwd(M, n, counts):
+    return sum(rw_batched_swiglu_bwd(M, n, counts))
+
+
+def bytes_rmsnorm_bwd(M, n):
+    return sum(rw_rmsnorm_bwd(M, n))
+
+
+def bytes_permute_pad_quant(n, counts):
+    return sum(rw_permute_pad_quant(n, counts))

@@ -63,6 +63,19 @@ int fq_version(void) { return 100; }
 
 const char* fq_last_error(void) { return g_err; }
 
+int fq_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink, int nontemporal,
+                 void* stream) {
+  const char* fn = "fq_stream_rw";
+  FQ_REQUIRE(read_bytes >= 0 && write_bytes >= 0 && read_bytes % 16 == 0 && write_bytes % 16 == 0, FQ_ERR_SHAPE,
+             "%s: byte counts must be non-negative multiples of 16", fn);
+  FQ_REQUIRE((read_bytes == 0 || (src && aligned16(src))) && (write_bytes == 0 || (dst && aligned16(dst))) && sink &&
+                 aligned16(sink),
+             FQ_ERR_ARG, "%s: NULL or misaligned pointer", fn);
+  return check_launch(fq::launch_stream_rw(src, read_bytes, dst, write_bytes, sink, nontemporal != 0,
+                                           (hipStream_t)stream),
+                      fn);
+}
+
 int fq_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t N,
                        int round_scale, int output_mode, int fp8_kind, void* stream) {
   const char* fn = "fq_blockwise_quant";

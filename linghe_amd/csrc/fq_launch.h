@@ -61,4 +61,8 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
                                        float* rstd, float* logits, void* q, float* s, int64_t M, int K, int N,
                                        float eps, int round_scale, int kind, hipStream_t stream);
 
+// measurement aid: read read_bytes from src, write write_bytes to dst (both multiples of 16), no arithmetic
+hipError_t launch_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,
+                            int nontemporal, hipStream_t stream);
+
 }  // namespace fq

@@ -44,8 +44,8 @@ template <int RPT>
 struct alignas(16) TileShared {
   uint8_t t[kGroup * kGroup];                       // transposed codes, 16-byte chunks XOR-swizzled
   float colmax[TileShape<RPT>::kWaves][kGroup];      // per-wave column amax
-  float2 cdiv[kGroup];                               // per column {scale, 1/scale}
-  float2 rdiv[kGroup];                               // per row    {scale, 1/scale}
+  float2 cdiv[kGroup];                               // per column the two terms of 1/scale (Divisor)
+  float2 rdiv[kGroup];                               // per row    the same
 };
 
 // Column maxima of a wave.  Lane (r, cg) = (lane >> 4, lane & 15) holds cm[j], the
@@ -182,7 +182,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       const float sc = make_scale<KIND, ROUND>(mine);
       const Divisor d = make_divisor(sc);
       const int i = rg * RPT + cg;
-      sh.rdiv[i] = make_float2(d.s, d.r);
+      sh.rdiv[i] = make_float2(d.r, d.rl);
       if (FULL || i < o.rows_valid) store_f32(s_base + (uint32_t)i, sc);  // a wave writes 4*RPT consecutive floats
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -192,8 +192,8 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
     for (int s = 0; s < RPT; ++s) {
       const float2 sr = sh.rdiv[rg * RPT + s];
       Divisor d;
-      d.s = sr.x;
-      d.r = sr.y;
+      d.r = sr.x;
+      d.rl = sr.y;
       float qv[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(v[s][j], d);
@@ -249,7 +249,7 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
       for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[w][tid]);
       const float sc = make_scale<KIND, ROUND>(m);
       const Divisor d = make_divisor(sc);
-      sh.cdiv[tid] = make_float2(d.s, d.r);
+      sh.cdiv[tid] = make_float2(d.r, d.rl);
       store_f32(st_base + (uint32_t)tid, sc);
     }
     __syncthreads();
@@ -260,8 +260,8 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
         const float4 a = src[h];
-        cd[2 * h].s = a.x; cd[2 * h].r = a.y;
-        cd[2 * h + 1].s = a.z; cd[2 * h + 1].r = a.w;
+        cd[2 * h].r = a.x; cd[2 * h].rl = a.y;
+        cd[2 * h + 1].r = a.z; cd[2 * h + 1].rl = a.w;
       }
     }
     // transposed codes -> LDS; byte (c, i) lives at c*128 + ((i>>4) ^ ((c>>3)&7))*16 + (i&15)

@@ -12,9 +12,9 @@ Acceptance (stricter than the reference's output_check):
     oracle, closer after an RMSNorm), so they differ from EACH OTHER by up to 6 ulp.
     The limits below are the largest differences measured over every shape here
     and the benchmark configurations:
-      - SwiGLU forward: none beyond 5 ulp, >= 98 % within 1 ulp (torch's CPU sigmoid
+      - SwiGLU forward: none beyond 5 ulp, >= 97 % within 1 ulp (99 % at the benchmark sizes) (torch's CPU sigmoid
         is 1/(1+exp(-x)) with a vectorised 2-ulp exp, the kernel's a hardware exp2);
-      - SwiGLU backward: none beyond 6 ulp, >= 98 % within 1 ulp, except where
+      - SwiGLU backward: none beyond 6 ulp, >= 97 % within 1 ulp (99 % at the benchmark sizes), except where
         dx1 = h*s + h*x1*(1-s)*s cancels (x1 near -1.28) in the element that makes a
         group's amax - a group of one or two rows of a ragged expert: there both
         sides must lie within that element's own error bound of the fp64 value;
@@ -37,8 +37,8 @@ from tests.helpers import (E4M3, E5M2, announce, check_quant_pair, gamma_bf16, g
 
 pytestmark = pytest.mark.gpu
 
-FUSED = dict(scale_max_ulp=5, scale_min_within1=0.98)        # SwiGLU forward
-FUSED_BWD = dict(scale_max_ulp=6, scale_min_within1=0.98)    # SwiGLU backward (+ the conditioned escape, see above)
+FUSED = dict(scale_max_ulp=5, scale_min_within1=0.97)        # SwiGLU forward
+FUSED_BWD = dict(scale_max_ulp=6, scale_min_within1=0.97)    # SwiGLU backward (+ the conditioned escape, see above)
 FUSED_NORM = dict(scale_max_ulp=6, scale_min_within1=0.9)    # RMSNorm vs pure oracle
 EXACT = dict(scale_max_ulp=0, scale_min_within1=1.0, min_identical=1.0)
 
