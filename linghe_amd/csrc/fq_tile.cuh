@@ -40,12 +40,13 @@ struct TileOut {
   int rows_valid;   // rows i < rows_valid exist (1..128)
 };
 
-template <int RPT>
+// NV: value tiles quantised together by one workgroup (2 in the SwiGLU backward: dx1, dx2)
+template <int RPT, int NV = 1>
 struct alignas(16) TileShared {
-  uint8_t t[kGroup * kGroup];                       // transposed codes, 16-byte chunks XOR-swizzled
-  float colmax[TileShape<RPT>::kWaves][kGroup];      // per-wave column amax
-  float2 cdiv[kGroup];                               // per column the two terms of 1/scale (Divisor)
-  float2 rdiv[kGroup];                               // per row    the same
+  uint8_t t[NV][kGroup * kGroup];                        // transposed codes, 16-byte chunks XOR-swizzled
+  float colmax[NV][TileShape<RPT>::kWaves][kGroup];       // per-wave column amax
+  float2 cdiv[NV][kGroup];                                // per column the two terms of 1/scale (Divisor)
+  float2 rdiv[NV][kGroup];                                // per row    the same
 };
 
 // Column maxima of a wave.  Lane (r, cg) = (lane >> 4, lane & 15) holds cm[j], the
@@ -125,40 +126,55 @@ __device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uin
   if (rem & 1) *(FQ_GLOBAL uint8_t*)(dst + p) = (uint8_t)(pick_dword(d0, d1, d2, d3, p >> 2) >> (8 * (p & 3)));
 }
 
-// Quantise the tile held in registers (v[s][j] = element (rg*RPT+s, cg*8+j);
-// rows >= rows_valid must hold 0).  All threads of the workgroup must call it.
-// FULL: the tile has all 128 rows, so no load or store needs a mask.
-template <int KIND, bool ROUND, int MODE, int RPT, bool FULL, int NT, bool LEAN>
-__device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], const TileOut& o,
-                                                   TileShared<RPT>& sh) {
+// Quantise NV tiles held in registers (v[t][s][j] = element (rg*RPT+s, cg*8+j) of tile t;
+// rows >= rows_valid must hold 0; the tiles share rows_valid).  All threads of the
+// workgroup must call it.  The tiles go through the column stage together: one set
+// of barriers for all of them, and the NV*128 column scales are computed by as many
+// threads at once.
+// FULL: the tiles have all 128 rows, so no load or store needs a mask.
+// TAIL_SYNC: end with a barrier (needed only when the shared memory is used again).
+template <int KIND, bool ROUND, int MODE, int RPT, bool FULL, int NT, bool LEAN, int NV, bool TAIL_SYNC>
+__device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8], const TileOut (&o)[NV],
+                                                    TileShared<RPT, NV>& sh) {
   using Shape = TileShape<RPT>;
+  static_assert(NV * kGroup <= Shape::kThreads, "one thread per column scale");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int cg = tid & 15;
   const int rg = tid >> 4;
+  const int rows_valid = o[0].rows_valid;
 
   // A wave owns 4*RPT consecutive rows.  In a partial tile the waves whose rows all
   // lie beyond the last stored row have nothing to quantise: their values are
   // zero, their row-wise outputs do not exist and their bytes of the transposed
   // tile are never stored, so they only keep the barriers company.
-  const bool live = FULL || wave * (4 * RPT) < o.rows_valid;
+  const bool live = FULL || wave * (4 * RPT) < rows_valid;
 
   // LEAN: the four output bases, which are the same in every lane, are moved to scalar
   // registers, so that each store is "scalar base + 32-bit lane offset" (a tile spans
   // at most 128 rows of at most 2^24 bytes) without 64-bit vector address arithmetic,
   // and the column maxima take the paired reduction: 10 % fewer vector instructions,
   // 3-9 % less time in every tile kernel but the plain blockwise quantiser.
-  uint8_t* q_base = o.q + o.q_off;
-  uint8_t* t_base = o.qt + o.t_off;
-  float* s_base = o.s + o.s_off;
-  float* st_base = o.st + o.st_off;
-  uint32_t q_ld = (uint32_t)o.q_ld, t_ld = (uint32_t)o.t_ld;
+  uint8_t* q_base[NV];
+  uint8_t* t_base[NV];
+  float* s_base[NV];
+  float* st_base[NV];
+  uint32_t q_ld = (uint32_t)o[0].q_ld, t_ld = (uint32_t)o[0].t_ld;
+#pragma unroll
+  for (int t = 0; t < NV; ++t) {
+    q_base[t] = o[t].q + o[t].q_off;
+    t_base[t] = o[t].qt + o[t].t_off;
+    s_base[t] = o[t].s + o[t].s_off;
+    st_base[t] = o[t].st + o[t].st_off;
+    if constexpr (LEAN) {
+      q_base[t] = (uint8_t*)uniform64((int64_t)q_base[t]);
+      t_base[t] = (uint8_t*)uniform64((int64_t)t_base[t]);
+      s_base[t] = (float*)uniform64((int64_t)s_base[t]);
+      st_base[t] = (float*)uniform64((int64_t)st_base[t]);
+    }
+  }
   if constexpr (LEAN) {
-    q_base = (uint8_t*)uniform64((int64_t)q_base);
-    t_base = (uint8_t*)uniform64((int64_t)t_base);
-    s_base = (float*)uniform64((int64_t)s_base);
-    st_base = (float*)uniform64((int64_t)st_base);
     q_ld = (uint32_t)uniform32((int)q_ld);
     t_ld = (uint32_t)uniform32((int)t_ld);
   }
@@ -166,151 +182,178 @@ __device__ __forceinline__ void quantize_tile_impl(const float (&v)[RPT][8], con
   // ------------------------------------------------------------- row-wise
   if ((MODE == 0 || MODE == 2) && live) {
     // every lane of a 16-lane row gets the amax of its RPT rows; lane cg < RPT then
-    // turns ONE of them (row rg*RPT+cg) into {scale, 1/scale}, stores the scale,
-    // and hands the pair to the other lanes through LDS.  The rows of a wave are
+    // turns ONE of them (row rg*RPT+cg) into its scale and divisor, stores the scale,
+    // and hands the divisor to the other lanes through LDS.  The rows of a wave are
     // written and read by that wave only, so no barrier is needed.
-    float mine = 0.f;
 #pragma unroll
-    for (int s = 0; s < RPT; ++s) {
-      float m = 0.f;
+    for (int t = 0; t < NV; ++t) {
+      float mine = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[s][j]));
-      m = row16_max(m);
-      if (cg == s) mine = m;
-    }
-    if (cg < RPT) {
-      const float sc = make_scale<KIND, ROUND>(mine);
-      const Divisor d = make_divisor(sc);
-      const int i = rg * RPT + cg;
-      sh.rdiv[i] = make_float2(d.r, d.rl);
-      if (FULL || i < o.rows_valid) store_f32(s_base + (uint32_t)i, sc);  // a wave writes 4*RPT consecutive floats
+      for (int s = 0; s < RPT; ++s) {
+        float m = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[t][s][j]));
+        m = row16_max(m);
+        if (cg == s) mine = m;
+      }
+      if (cg < RPT) {
+        const float sc = make_scale<KIND, ROUND>(mine);
+        const Divisor d = make_divisor(sc);
+        const int i = rg * RPT + cg;
+        sh.rdiv[t][i] = make_float2(d.r, d.rl);
+        if (FULL || i < rows_valid) store_f32(s_base[t] + (uint32_t)i, sc);  // a wave writes 4*RPT consecutive floats
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int s = 0; s < RPT; ++s) {
-      const float2 sr = sh.rdiv[rg * RPT + s];
-      Divisor d;
-      d.r = sr.x;
-      d.rl = sr.y;
-      float qv[8];
+    for (int t = 0; t < NV; ++t) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(v[s][j], d);
-      uint2 pk;
-      pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-      pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
-      const int i = rg * RPT + s;
-      if (FULL || i < o.rows_valid) store8<(NT & 2) != 0>(q_base + ((uint32_t)i * q_ld + (uint32_t)cg * 8u), pk);
+      for (int s = 0; s < RPT; ++s) {
+        const float2 sr = sh.rdiv[t][rg * RPT + s];
+        Divisor d;
+        d.r = sr.x;
+        d.rl = sr.y;
+        float qv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(v[t][s][j], d);
+        uint2 pk;
+        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+        const int i = rg * RPT + s;
+        if (FULL || i < rows_valid) store8<(NT & 2) != 0>(q_base[t] + ((uint32_t)i * q_ld + (uint32_t)cg * 8u), pk);
+      }
     }
   }
 
   // ---------------------------------------------------------- column-wise
   if constexpr (MODE == 1 || MODE == 2) {
-    float cm[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) cm[j] = 0.f;
-    if constexpr (LEAN) {
-      float cm_lo = 0.f, cm_hi = 0.f;
-      if (live) {
+    for (int t = 0; t < NV; ++t) {
+      float cm[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          float m = 0.f;
+      for (int j = 0; j < 8; ++j) cm[j] = 0.f;
+      if constexpr (LEAN) {
+        float cm_lo = 0.f, cm_hi = 0.f;
+        if (live) {
 #pragma unroll
-          for (int s = 0; s < RPT; ++s) m = fmaxf(m, fabsf(v[s][j]));
-          cm[j] = m;
+          for (int j = 0; j < 8; ++j) {
+            float m = 0.f;
+#pragma unroll
+            for (int s = 0; s < RPT; ++s) m = fmaxf(m, fabsf(v[t][s][j]));
+            cm[j] = m;
+          }
+          wave_column_max(cm, cm_lo, cm_hi);
         }
-        wave_column_max(cm, cm_lo, cm_hi);
-      }
-      const int r = lane >> 4;
-      float* dst = &sh.colmax[wave][cg * 8 + (((r & 1) << 1) | (r >> 1))];
-      dst[0] = cm_lo;
-      dst[4] = cm_hi;
-    } else {
-      if (live) {
+        const int r = lane >> 4;
+        float* dst = &sh.colmax[t][wave][cg * 8 + (((r & 1) << 1) | (r >> 1))];
+        dst[0] = cm_lo;
+        dst[4] = cm_hi;
+      } else {
+        if (live) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          float m = 0.f;
+          for (int j = 0; j < 8; ++j) {
+            float m = 0.f;
 #pragma unroll
-          for (int s = 0; s < RPT; ++s) m = fmaxf(m, fabsf(v[s][j]));
-          cm[j] = max_across_rows(m);
+            for (int s = 0; s < RPT; ++s) m = fmaxf(m, fabsf(v[t][s][j]));
+            cm[j] = max_across_rows(m);
+          }
         }
-      }
-      if (lane < 16) {
-        float4* dst = (float4*)&sh.colmax[wave][cg * 8];
-        dst[0] = make_float4(cm[0], cm[1], cm[2], cm[3]);
-        dst[1] = make_float4(cm[4], cm[5], cm[6], cm[7]);
+        if (lane < 16) {
+          float4* dst = (float4*)&sh.colmax[t][wave][cg * 8];
+          dst[0] = make_float4(cm[0], cm[1], cm[2], cm[3]);
+          dst[1] = make_float4(cm[4], cm[5], cm[6], cm[7]);
+        }
       }
     }
     __syncthreads();
-    if (tid < kGroup) {
-      float m = sh.colmax[0][tid];
+    if (tid < NV * kGroup) {  // thread (t, c): the scale of column c of tile t
+      const int t = tid / kGroup, c = tid % kGroup;
+      float m = sh.colmax[t][0][c];
 #pragma unroll
-      for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[w][tid]);
+      for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[t][w][c]);
       const float sc = make_scale<KIND, ROUND>(m);
       const Divisor d = make_divisor(sc);
-      sh.cdiv[tid] = make_float2(d.r, d.rl);
-      store_f32(st_base + (uint32_t)tid, sc);
+      sh.cdiv[t][c] = make_float2(d.r, d.rl);
+      float* dst = st_base[0];
+#pragma unroll
+      for (int u = 1; u < NV; ++u) dst = (t == u) ? st_base[u] : dst;
+      store_f32(dst + (uint32_t)c, sc);
     }
     __syncthreads();
     if (live) {
-    Divisor cd[8];
-    {
-      const float4* src = (const float4*)&sh.cdiv[cg * 8];
 #pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const float4 a = src[h];
-        cd[2 * h].r = a.x; cd[2 * h].rl = a.y;
-        cd[2 * h + 1].r = a.z; cd[2 * h + 1].rl = a.w;
+      for (int t = 0; t < NV; ++t) {
+        Divisor cd[8];
+        {
+          const float4* src = (const float4*)&sh.cdiv[t][cg * 8];
+#pragma unroll
+          for (int h = 0; h < 4; ++h) {
+            const float4 a = src[h];
+            cd[2 * h].r = a.x; cd[2 * h].rl = a.y;
+            cd[2 * h + 1].r = a.z; cd[2 * h + 1].rl = a.w;
+          }
+        }
+        // transposed codes -> LDS; byte (c, i) lives at c*128 + ((i>>4) ^ ((c>>3)&7))*16 + (i&15)
+        const int i0 = rg * RPT;
+        const int chunk = (i0 >> 4) ^ (cg & 7);
+        uint8_t* base = sh.t[t] + chunk * 16 + (i0 & 15);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const Divisor d = cd[j];
+          float qv[RPT];
+#pragma unroll
+          for (int s = 0; s < RPT; ++s) qv[s] = div_by_scale<ROUND>(v[t][s][j], d);
+          uint8_t* p = base + (cg * 8 + j) * kGroup;
+          if constexpr (RPT == 8) {
+            uint2 pk;
+            pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+            pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+            *(uint2*)p = pk;
+          } else {
+            *(uint32_t*)p = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+          }
+        }
       }
-    }
-    // transposed codes -> LDS; byte (c, i) lives at c*128 + ((i>>4) ^ ((c>>3)&7))*16 + (i&15)
-    const int i0 = rg * RPT;
-    const int chunk = (i0 >> 4) ^ (cg & 7);
-    uint8_t* base = sh.t + chunk * 16 + (i0 & 15);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const Divisor d = cd[j];
-      float qv[RPT];
-#pragma unroll
-      for (int s = 0; s < RPT; ++s) qv[s] = div_by_scale<ROUND>(v[s][j], d);
-      uint8_t* p = base + (cg * 8 + j) * kGroup;
-      if constexpr (RPT == 8) {
-        uint2 pk;
-        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
-        *(uint2*)p = pk;
-      } else {
-        *(uint32_t*)p = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-      }
-    }
     }
     __syncthreads();
     // each transposed row (one column, 128 row-bytes) leaves as 8 x 16 bytes
     constexpr int kRowsPerPass = Shape::kThreads / 8;
     const int ch = tid & 7;
 #pragma unroll
-    for (int k = 0; k < kGroup / kRowsPerPass; ++k) {
-      const int c = (tid >> 3) + k * kRowsPerPass;
-      if constexpr (FULL) {
-        const uint4 val = *(const uint4*)(sh.t + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
-        store16_any<(NT & 1) != 0>(t_base + ((uint32_t)c * t_ld + (uint32_t)ch * 16u), val);
-      } else {
-        store_t_row<(NT & 1) != 0>(sh.t + c * kGroup, (c >> 3) & 7, t_base + (uint32_t)c * t_ld, o.rows_valid, ch);
+    for (int t = 0; t < NV; ++t) {
+#pragma unroll
+      for (int k = 0; k < kGroup / kRowsPerPass; ++k) {
+        const int c = (tid >> 3) + k * kRowsPerPass;
+        if constexpr (FULL) {
+          const uint4 val = *(const uint4*)(sh.t[t] + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
+          store16_any<(NT & 1) != 0>(t_base[t] + ((uint32_t)c * t_ld + (uint32_t)ch * 16u), val);
+        } else {
+          store_t_row<(NT & 1) != 0>(sh.t[t] + c * kGroup, (c >> 3) & 7, t_base[t] + (uint32_t)c * t_ld, rows_valid, ch);
+        }
       }
     }
-    __syncthreads();  // LDS is reused by a following call
+    if constexpr (TAIL_SYNC) __syncthreads();  // LDS is reused by a following call
   }
 }
 
 // NT: bit 0 = transposed codes, bit 1 = row-wise codes leave with the non-temporal hint
-template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0, bool LEAN = true>
-__device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o,
-                                              TileShared<RPT>& sh) {
+template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0, bool LEAN = true, int NV = 1, bool TAIL_SYNC = false>
+__device__ __forceinline__ void quantize_tiles(const float (&v)[NV][RPT][8], const TileOut (&o)[NV],
+                                               TileShared<RPT, NV>& sh) {
   // workgroup-uniform choice of the mask-free path
-  const bool full = o.rows_valid == kGroup;
-  if (full) quantize_tile_impl<KIND, ROUND, MODE, RPT, true, NT, LEAN>(v, o, sh);
-  else quantize_tile_impl<KIND, ROUND, MODE, RPT, false, NT, LEAN>(v, o, sh);
+  const bool full = o[0].rows_valid == kGroup;
+  if (full) quantize_tiles_impl<KIND, ROUND, MODE, RPT, true, NT, LEAN, NV, TAIL_SYNC>(v, o, sh);
+  else quantize_tiles_impl<KIND, ROUND, MODE, RPT, false, NT, LEAN, NV, TAIL_SYNC>(v, o, sh);
+}
+
+// one tile
+template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0, bool LEAN = true>
+__device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o, TileShared<RPT>& sh) {
+  const float (&vs)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(v);
+  const TileOut (&os)[1] = reinterpret_cast<const TileOut (&)[1]>(o);
+  quantize_tiles<KIND, ROUND, MODE, RPT, NT, LEAN, 1, false>(vs, os, sh);
 }
 
 // ---------------------------------------------------------------------------
