@@ -70,7 +70,7 @@ def build_cases(names, dev):
             cases[name] = kw
 
     # ---------------------------------------------------------------- cfg1 / cfg5b / cfg5c
-    def rms_quant_case(name, data, mode):
+    def rms_quant_case(name, data, mode, pow2=False):
         x_cpu, g_cpu, eps = data["x"], data["gamma"], data["eps"]
         M, n = x_cpu.shape
         gd = g_cpu.to(dev)
@@ -93,7 +93,7 @@ def build_cases(names, dev):
             else:
                 s["qt"], s["st"] = None, None
             s["args"] = (_p(s["x"]), _p(gd), _p(s["q"]), _p(s["s"]), _p(s["rstd"]), _p(s["qt"]), _p(s["st"]),
-                         M, n, float(eps), 0, mode, _lib.FQ_E4M3, stream)
+                         M, n, float(eps), int(pow2), mode, _lib.FQ_E4M3, stream)
             return s
 
         def launch(s):
@@ -101,11 +101,13 @@ def build_cases(names, dev):
 
         def cpu_fn():
             from oracle import fq_oracle as O
-            return O.rms_norm_and_block_quant_forward(x_cpu, g_cpu, eps, False)
+            return O.rms_norm_and_block_quant_forward(x_cpu, g_cpu, eps, pow2)
 
         label = "triton_rms_norm_and_block_quant_forward(output_mode=%d)" % mode
         if mode == 2:
             label += " two passes"
+        if pow2:
+            label += ", round_scale=True"
         return Case(name, label, [M, n],
                     configs.rw_rmsnorm_quant(M, n, mode), make_set, launch, cpu_fn)
 
@@ -117,11 +119,14 @@ def build_cases(names, dev):
         return lazy["cfg5"]
 
     add("cfg1", build=lambda: rms_quant_case("cfg1", configs.cfg1_rmsnorm_quant(), 2))
+    # the same with power-of-two scales: what the autograd callers request when the
+    # quantizer's recipe sets force_pow_2_scales (linghe/facade/norm.py:62-69)
+    add("cfg1_pow2", build=lambda: rms_quant_case("cfg1_pow2", configs.cfg1_rmsnorm_quant(), 2, True))
     add("cfg5b", build=lambda: rms_quant_case("cfg5b", cfg5(), 2))
     add("cfg5c", build=lambda: rms_quant_case("cfg5c", cfg5(), 1))
 
     # ---------------------------------------------------------------- cfg2
-    def swiglu_fwd_case():
+    def swiglu_fwd_case(name="cfg2", pow2=False):
         x_cpu = configs.cfg2_swiglu_fwd()["x"]
         M, N = x_cpu.shape
         n = N // 2
@@ -131,7 +136,7 @@ def build_cases(names, dev):
                      s=torch.empty((n // 128, M), device=dev, dtype=torch.float32),
                      qt=torch.empty((n, M), device=dev, dtype=FP8),
                      st=torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32))
-            s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, 0, 2,
+            s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, int(pow2), 2,
                          _lib.FQ_E4M3, stream)
             return s
 
@@ -140,12 +145,14 @@ def build_cases(names, dev):
 
         def cpu_fn():
             from oracle import fq_oracle as O
-            return O.silu_and_block_quant_forward(x_cpu, False)
+            return O.silu_and_block_quant_forward(x_cpu, pow2)
 
-        return Case("cfg2", "triton_silu_and_block_quant_forward(output_mode=2)", [M, N],
+        return Case(name, "triton_silu_and_block_quant_forward(output_mode=2%s)" % (", round_scale=True" if pow2 else ""),
+                    [M, N],
                     configs.rw_swiglu_fwd(M, n), make_set, launch, cpu_fn)
 
     add("cfg2", build=swiglu_fwd_case)
+    add("cfg2_pow2", build=lambda: swiglu_fwd_case("cfg2_pow2", True))
 
     # ---------------------------------------------------------------- cfg3 (+ backward)
     def batched_case(backward):
@@ -201,7 +208,7 @@ def build_cases(names, dev):
     add("cfg3b", build=lambda: batched_case(True))
 
     # ---------------------------------------------------------------- cfg4
-    def swiglu_bwd_case(kind, name):
+    def swiglu_bwd_case(kind, name, pow2=False):
         d = lazy.setdefault("cfg4", configs.cfg4_swiglu_bwd())
         dy_cpu, x_cpu = d["dy"], d["x"]
         M, N = x_cpu.shape
@@ -213,8 +220,8 @@ def build_cases(names, dev):
                      s=torch.empty((N // 128, M), device=dev, dtype=torch.float32),
                      qt=torch.empty((N, M), device=dev, dtype=dt),
                      st=torch.empty((M // 128, N), device=dev, dtype=torch.float32))
-            s["args"] = (_p(s["dy"]), _p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, 0, kind,
-                         stream)
+            s["args"] = (_p(s["dy"]), _p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, int(pow2),
+                         kind, stream)
             return s
 
         def launch(s):
@@ -222,13 +229,16 @@ def build_cases(names, dev):
 
         def cpu_fn():
             from oracle import fq_oracle as O
-            return O.silu_and_block_quant_backward(dy_cpu, x_cpu, False, dt)
+            return O.silu_and_block_quant_backward(dy_cpu, x_cpu, pow2, dt)
 
-        return Case(name, "triton_silu_and_block_quant_backward(fp8=%s)" % str(dt).split(".")[-1], [M, N],
+        return Case(name, "triton_silu_and_block_quant_backward(fp8=%s%s)" % (str(dt).split(".")[-1],
+                                                                               ", round_scale=True" if pow2 else ""),
+                    [M, N],
                     configs.rw_swiglu_bwd(M, n), make_set, launch, cpu_fn)
 
     add("cfg4", build=lambda: swiglu_bwd_case(_lib.FQ_E4M3, "cfg4"))
     add("cfg4_e5m2", build=lambda: swiglu_bwd_case(_lib.FQ_E5M2, "cfg4_e5m2"))
+    add("cfg4_pow2", build=lambda: swiglu_bwd_case(_lib.FQ_E4M3, "cfg4_pow2", True))
 
     # ---------------------------------------------------------------- cfg5a
     def rms_bwd_case():
@@ -501,6 +511,7 @@ def load_traffic_table():
 
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
+       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router",
        "stream_read", "stream_copy"]
 

@@ -132,6 +132,21 @@ __device__ __forceinline__ uint32_t pack4_fp8(float a, float b, float c, float d
   return w;
 }
 
+typedef short i16x2_t __attribute__((ext_vector_type(2)));
+// codes of a/s, b/s, c/s, d/s for a power-of-two s (exact quotients, RNE)
+template <int KIND>
+__device__ __forceinline__ uint32_t pack4_fp8_scaled(float a, float b, float c, float d, float s) {
+  i16x2_t w = __builtin_bit_cast(i16x2_t, as_u32(a));
+  if constexpr (!Fp8Traits<KIND>::kBf8) {
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, a, b, s, false);
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, c, d, s, true);
+  } else {
+    w = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(w, a, b, s, false);
+    w = __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(w, c, d, s, true);
+  }
+  return __builtin_bit_cast(uint32_t, w);
+}
+
 // ---------------------------------------------------------------------------
 // Division by a scale that is shared by many elements, in two operations each.
 //   per scale:   r  = 1/s, v_rcp_f32 plus one Newton step
@@ -158,12 +173,48 @@ __device__ __forceinline__ Divisor make_divisor(float s) {
   d.rl = __builtin_fmaf(-s, r, 1.0f) * r;
   return d;
 }
-// POW2: the scale is a power of two, its reciprocal is exact and so is the
-// product v * (1/s): one multiplication IS the division
-template <bool POW2>
 __device__ __forceinline__ float div_by_scale(float v, const Divisor& d) {
-  if constexpr (POW2) return v * d.r;
-  else return __builtin_fmaf(v, d.r, v * d.rl);
+  return __builtin_fmaf(v, d.r, v * d.rl);
+}
+
+// What the quantisers keep per scale.  POW2 (round_scale): the scale is a power of two
+// and rides in the convert instruction itself (v_cvt_scalef32_pk_*: codes of v / scale,
+// only the exponent of the scale operand is used), so there is no arithmetic per
+// element at all; otherwise the two terms of the reciprocal.
+template <bool POW2>
+struct Quantum {
+  float a, b;  // POW2: a = scale;  else {a, b} = Divisor{r, rl}
+};
+template <bool POW2>
+__device__ __forceinline__ Quantum<POW2> make_quantum(float s) {
+  Quantum<POW2> q;
+  if constexpr (POW2) {
+    q.a = s;
+    q.b = 0.f;
+  } else {
+    const Divisor d = make_divisor(s);
+    q.a = d.r;
+    q.b = d.rl;
+  }
+  return q;
+}
+
+// codes of four values under one scale
+template <int KIND, bool POW2>
+__device__ __forceinline__ uint32_t quantize4(float a, float b, float c, float d, const Quantum<POW2>& q) {
+  if constexpr (POW2) {
+    return pack4_fp8_scaled<KIND>(a, b, c, d, q.a);
+  } else {
+    const Divisor dv{q.a, q.b};
+    return pack4_fp8<KIND>(div_by_scale(a, dv), div_by_scale(b, dv), div_by_scale(c, dv), div_by_scale(d, dv));
+  }
+}
+template <int KIND, bool POW2>
+__device__ __forceinline__ uint2 quantize8(const float (&v)[8], const Quantum<POW2>& q) {
+  uint2 pk;
+  pk.x = quantize4<KIND, POW2>(v[0], v[1], v[2], v[3], q);
+  pk.y = quantize4<KIND, POW2>(v[4], v[5], v[6], v[7], q);
+  return pk;
 }
 
 // exp2(ceil(log2(s))) as torch evaluates it in fp32 (linghe/tools/util.py:61-62):

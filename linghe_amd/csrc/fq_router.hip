@@ -186,22 +186,16 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
       }
       m = row16_max(m);
       const float sc = make_scale<KIND, ROUND>(m);
-      const Divisor d = make_divisor(sc);
       const uint4 hi = pack8_bf16(yv);
-      float back[8], lo[8], qv[8];
+      float back[8], lo[8];
       unpack8(hi, back);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        lo[i] = yv[i] - back[i];
-        qv[i] = div_by_scale<ROUND>(yv[i], d);
-      }
+      for (int i = 0; i < 8; ++i) lo[i] = yv[i] - back[i];
       const int slot = ahalf * 32 + ((RPT * rg + u) ^ aj);
       sh.a[buf][0][aj][slot] = hi;
       sh.a[buf][1][aj][slot] = pack8_bf16(lo);
       store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, hi);
-      uint2 pk;
-      pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-      pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+      const uint2 pk = quantize8<KIND, ROUND>(yv, make_quantum<ROUND>(sc));
       store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
       if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
     }
@@ -404,7 +398,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
       unpack8(sgamma[kb * 16 + cg], g);
 #pragma unroll
       for (int u = 0; u < RPT; ++u) {
-        float a[8], yv[8], qv[8];
+        float a[8], yv[8];
         unpack8(xr[kb][u], a);
         float m = 0.f;
 #pragma unroll
@@ -414,13 +408,8 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
         }
         m = row16_max(m);
         const float sc = make_scale<KIND, ROUND>(m);
-        const Divisor d = make_divisor(sc);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) qv[i] = div_by_scale<ROUND>(yv[i], d);
         store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, pack8_bf16(yv));
-        uint2 pk;
-        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+        const uint2 pk = quantize8<KIND, ROUND>(yv, make_quantum<ROUND>(sc));
         store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
         if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
       }

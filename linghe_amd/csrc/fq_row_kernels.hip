@@ -180,13 +180,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
         for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(y[j]));
         m = row16_max(m);
         const float sc = make_scale<KIND, ROUND>(m);
-        const Divisor d = make_divisor(sc);
-        float qv[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(y[j], d);
-        uint2 pk;
-        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+        const uint2 pk = quantize8<KIND, ROUND>(y, make_quantum<ROUND>(sc));
         if (c * 8 < n) {
           st8((uint8_t*)out + row * n + c * 8, pk);
           if ((c & 15) == 0) scale[(int64_t)(c >> 4) * M + row] = sc;
@@ -505,13 +499,7 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __rest
     for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(a[j]));
     m = row16_max(m);
     const float sc = make_scale<KIND, ROUND>(m);
-    const Divisor d = make_divisor(sc);
-    float qv[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(a[j], d);
-    uint2 pk;
-    pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-    pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+    const uint2 pk = quantize8<KIND, ROUND>(a, make_quantum<ROUND>(sc));
     if (ok) {
       st8(q + g * kGroup + sub * 8, pk);
       if (sub == 0) s[g] = sc;
@@ -868,17 +856,13 @@ __global__ __launch_bounds__(256) void block_quant_kernel(const uint16_t* __rest
   __syncthreads();
   m = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
   const float sc = make_scale<KIND, ROUND>(m);
-  const Divisor d = make_divisor(sc);
+  const Quantum<ROUND> d = make_quantum<ROUND>(sc);
   if (threadIdx.x == 0) s[(int64_t)rb * ncb + cb] = sc;
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
-    float a[8], qv[8];
+    float a[8];
     unpack8(raw[k], a);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(a[j], d);
-    uint2 pk;
-    pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-    pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+    const uint2 pk = quantize8<KIND, ROUND>(a, d);
     st8(dst + (off + (uint32_t)k * (uint32_t)N), pk);
   }
 }

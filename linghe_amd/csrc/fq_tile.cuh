@@ -45,7 +45,7 @@ template <int RPT, int NV = 1>
 struct alignas(16) TileShared {
   uint8_t t[NV][kGroup * kGroup];                        // transposed codes, 16-byte chunks XOR-swizzled
   float colmax[NV][TileShape<RPT>::kWaves][kGroup];       // per-wave column amax
-  float2 cdiv[NV][kGroup];                                // per column the two terms of 1/scale (Divisor)
+  float2 cdiv[NV][kGroup];                                // per column what the quantiser keeps per scale (Quantum)
   float2 rdiv[NV][kGroup];                                // per row    the same
 };
 
@@ -198,9 +198,9 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
       }
       if (cg < RPT) {
         const float sc = make_scale<KIND, ROUND>(mine);
-        const Divisor d = make_divisor(sc);
+        const Quantum<ROUND> d = make_quantum<ROUND>(sc);
         const int i = rg * RPT + cg;
-        sh.rdiv[t][i] = make_float2(d.r, d.rl);
+        sh.rdiv[t][i] = make_float2(d.a, d.b);
         if (FULL || i < rows_valid) store_f32(s_base[t] + (uint32_t)i, sc);  // a wave writes 4*RPT consecutive floats
       }
     }
@@ -212,15 +212,8 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
 #pragma unroll
       for (int s = 0; s < RPT; ++s) {
         const float2 sr = sh.rdiv[t][rg * RPT + s];
-        Divisor d;
-        d.r = sr.x;
-        d.rl = sr.y;
-        float qv[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) qv[j] = div_by_scale<ROUND>(v[t][s][j], d);
-        uint2 pk;
-        pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-        pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+        const Quantum<ROUND> d{sr.x, sr.y};
+        const uint2 pk = quantize8<KIND, ROUND>(v[t][s], d);
         const int i = rg * RPT + s;
         if (FULL || i < rows_valid) store8<(NT & 2) != 0>(q_base[t] + ((uint32_t)i * q_ld + (uint32_t)cg * 8u), pk);
       }
@@ -274,8 +267,8 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
 #pragma unroll
       for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[t][w][c]);
       const float sc = make_scale<KIND, ROUND>(m);
-      const Divisor d = make_divisor(sc);
-      sh.cdiv[t][c] = make_float2(d.r, d.rl);
+      const Quantum<ROUND> d = make_quantum<ROUND>(sc);
+      sh.cdiv[t][c] = make_float2(d.a, d.b);
       float* dst = st_base[0];
 #pragma unroll
       for (int u = 1; u < NV; ++u) dst = (t == u) ? st_base[u] : dst;
@@ -285,14 +278,14 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
     if (live) {
 #pragma unroll
       for (int t = 0; t < NV; ++t) {
-        Divisor cd[8];
+        Quantum<ROUND> cd[8];
         {
           const float4* src = (const float4*)&sh.cdiv[t][cg * 8];
 #pragma unroll
           for (int h = 0; h < 4; ++h) {
             const float4 a = src[h];
-            cd[2 * h].r = a.x; cd[2 * h].rl = a.y;
-            cd[2 * h + 1].r = a.z; cd[2 * h + 1].rl = a.w;
+            cd[2 * h].a = a.x; cd[2 * h].b = a.y;
+            cd[2 * h + 1].a = a.z; cd[2 * h + 1].b = a.w;
           }
         }
         // transposed codes -> LDS; byte (c, i) lives at c*128 + ((i>>4) ^ ((c>>3)&7))*16 + (i&15)
@@ -301,18 +294,15 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
         uint8_t* base = sh.t[t] + chunk * 16 + (i0 & 15);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const Divisor d = cd[j];
-          float qv[RPT];
-#pragma unroll
-          for (int s = 0; s < RPT; ++s) qv[s] = div_by_scale<ROUND>(v[t][s][j], d);
+          const Quantum<ROUND> d = cd[j];
           uint8_t* p = base + (cg * 8 + j) * kGroup;
           if constexpr (RPT == 8) {
             uint2 pk;
-            pk.x = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
-            pk.y = pack4_fp8<KIND>(qv[4], qv[5], qv[6], qv[7]);
+            pk.x = quantize4<KIND, ROUND>(v[t][0][j], v[t][1][j], v[t][2][j], v[t][3][j], d);
+            pk.y = quantize4<KIND, ROUND>(v[t][4][j], v[t][5][j], v[t][6][j], v[t][7][j], d);
             *(uint2*)p = pk;
           } else {
-            *(uint32_t*)p = pack4_fp8<KIND>(qv[0], qv[1], qv[2], qv[3]);
+            *(uint32_t*)p = quantize4<KIND, ROUND>(v[t][0][j], v[t][1][j], v[t][2][j], v[t][3][j], d);
           }
         }
       }

@@ -185,3 +185,57 @@ def test_cfg5_rmsnorm_large_full(gpu):
     torch.cuda.synchronize()
     assert torch.equal((dx.float() * 2).cpu(), dx2.float().cpu())
     assert torch.equal((dg * 2).cpu(), dg2.cpu())
+
+
+def test_reference_batched_shape_32_experts(gpu):
+    """The reference's own largest batched case (tests/test_silu.py:730-741): 32 experts of
+    1024..3072 rows (multiples of 16), 8192-wide input.  The whole problem runs on the GPU;
+    the oracle checks four experts (first, second, the smallest and the last), whose outputs
+    are independent slices of the packed layouts, forward and backward."""
+    import random
+
+    from linghe_amd.utils.silu import (triton_batch_weighted_silu_and_block_quant_backward as bwd,
+                                       triton_batch_weighted_silu_and_block_quant_forward as fwd)
+
+    announce("reference batched shape: 32 experts x ~2048 rows x 8192")
+    rnd = random.Random(7)
+    M0, N, E = 2048, 8192, 32
+    counts = [rnd.randint(M0 // 2, M0 // 2 * 3) // 16 * 16 for _ in range(E)]
+    bs, n = sum(counts), N // 2
+    g = torch.Generator().manual_seed(735)
+    x = torch.empty(bs, N, dtype=torch.bfloat16)
+    for r0 in range(0, bs, 8192):  # in slabs, to bound host memory
+        x[r0:r0 + 8192] = torch.randn(min(8192, bs - r0), N, generator=g).to(torch.bfloat16)
+    x[:3] = 0.0
+    w = torch.randn(bs, 1, generator=g)
+    dy = torch.empty(bs, n, dtype=torch.bfloat16)
+    for r0 in range(0, bs, 8192):
+        dy[r0:r0 + 8192] = torch.randn(min(8192, bs - r0), n, generator=g).to(torch.bfloat16)
+    cnt = torch.tensor(counts, dtype=torch.int32, device=gpu)
+    xd, wd, dyd = x.to(gpu), w.to(gpu), dy.to(gpu)
+    q, s, qt, st = fwd(xd, wd, cnt, counts, output_mode=2)
+    dq, ds, dw, dqt, dst = bwd(dyd, xd, wd, cnt, splits=counts)
+    torch.cuda.synchronize()
+    assert q.shape == (bs, n) and dq.shape == (bs, N) and dw.shape == (bs, 1)
+    q, s, qt, st = q.cpu(), s.cpu().view(-1), qt.cpu().view(-1), st.cpu().view(-1)
+    dq, ds, dw, dqt, dst = dq.cpu(), ds.cpu().view(-1), dw.cpu(), dqt.cpu().view(-1), dst.cpu().view(-1)
+    starts = [sum(counts[:e]) for e in range(E)]
+    tblocks = [sum((c + 127) // 128 for c in counts[:e]) for e in range(E)]
+    for e in sorted({0, 1, counts.index(min(counts)), E - 1}):
+        si, ce, tb = starts[e], counts[e], tblocks[e]
+        nblk = (ce + 127) // 128
+        xe, we, dye = x[si:si + ce], w[si:si + ce], dy[si:si + ce]
+        ref = O.batch_weighted_silu_and_block_quant_forward(xe, we, [ce], False)
+        check_quant_pair(f"ref32.e{e}.row", ref[0], ref[1], q[si:si + ce], s[si * (n // 128):(si + ce) * (n // 128)],
+                         **FUSED)
+        check_quant_pair(f"ref32.e{e}.col", ref[2], ref[3], qt[si * n:(si + ce) * n], st[tb * n:(tb + nblk) * n],
+                         **FUSED)
+        rb = O.batch_weighted_silu_and_block_quant_backward(dye, xe, we, [ce], False)
+        check_quant_pair(f"ref32.e{e}.bwd.row", rb[0], rb[1], dq[si:si + ce],
+                         ds[si * (N // 128):(si + ce) * (N // 128)], **FUSED_BWD)
+        check_quant_pair(f"ref32.e{e}.bwd.col", rb[3], rb[4], dqt[si * N:(si + ce) * N],
+                         dst[tb * N:(tb + nblk) * N], **FUSED_BWD)
+        torch.testing.assert_close(dw[si:si + ce], rb[2], rtol=1e-4, atol=1e-4 * float(rb[2].abs().max()))
+    # every 1x128 group of every expert reaches the format's maximum: no group was skipped or
+    # mis-scaled (the first three rows are zero rows)
+    _group_max_is_fmax(q[3:], torch.ones(bs - 3, n // 128), 448.0, "ref32 row groups")
