@@ -374,7 +374,7 @@ def build_cases(names, dev):
                      q=torch.empty((M, K), device=dev, dtype=FP8),
                      s=torch.empty((K // 128, M), device=dev, dtype=torch.float32))
             s["ws"] = torch.empty_like(rwd)
-            s["args"] = (_p(s["x"]), _p(nwd), _p(rwd), _p(s["ws"]), _p(s["y"]), _p(s["r"]), _p(s["lg"]), _p(s["q"]), _p(s["s"]),
+            s["args"] = (_p(s["x"]), _p(nwd), _p(rwd), 0, _p(s["ws"]), _p(s["y"]), _p(s["r"]), _p(s["lg"]), _p(s["q"]), _p(s["s"]),
                          M, K, N, 1e-6, 0, _lib.FQ_E4M3, stream)
             return s
 

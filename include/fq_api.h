@@ -145,16 +145,24 @@ int fq_rmsnorm_quant_fwd(const void* x, const void* gamma, void* q, float* s, fl
                          int64_t M, int64_t n, float eps, int round_scale, int output_mode, int fp8_kind,
                          void* stream);
 
+/* bytes of weight_scratch fq_rmsnorm_router_quant_fwd needs: N*K*2 for a bf16 router
+ * weight, N*K*4 for an fp32 one (0 for sizes the entry point refuses) */
+int64_t fq_rmsnorm_router_scratch_bytes(int64_t K, int64_t N, int weight_is_fp32);
+
 /* triton_rms_norm_fp32_gemm_block_quant_forward, output_mode 0,
  * linghe/utils/norm.py:690-784 (kernel :616-687).  x bf16 [M,K], gamma bf16 [K],
- * route_weight bf16 [N,K] (N = 128, 256, 384 or 512), M a multiple of 32.
- * Writes y bf16 [M,K] (the normalised x), rstd [M], logits fp32 [M,N] = y_fp32 @
- * route_weight^T, q [M,K] and s [K/128, M].  weight_scratch: N*K*2 bytes the
- * call overwrites (route_weight re-ordered for the matrix cores).
+ * route_weight [N,K] bf16 or (weight_is_fp32) fp32, N a multiple of 128 up to
+ * 8192, M a multiple of 32.  Writes y bf16 [M,K] (the normalised x), rstd [M],
+ * logits fp32 [M,N] = y_fp32 @ route_weight^T, q [M,K] and s [K/128, M].
+ * The product has fp32-GEMM accuracy: y, and an fp32 weight, enter the matrix
+ * cores as two bf16 terms each (16 significant bits; the reference's tl.dot on
+ * fp32 operands uses fewer).  weight_scratch: fq_rmsnorm_router_scratch_bytes()
+ * bytes the call overwrites (the weight re-ordered for the matrix cores).
  * (output_mode 1 of the reference is fq_rmsnorm_quant_fwd with output_mode 1.) */
-int fq_rmsnorm_router_quant_fwd(const void* x, const void* gamma, const void* route_weight, void* weight_scratch,
-                                void* y, float* rstd, float* logits, void* q, float* s, int64_t M, int64_t K,
-                                int64_t N, float eps, int round_scale, int fp8_kind, void* stream);
+int fq_rmsnorm_router_quant_fwd(const void* x, const void* gamma, const void* route_weight, int weight_is_fp32,
+                                void* weight_scratch, void* y, float* rstd, float* logits, void* q, float* s,
+                                int64_t M, int64_t K, int64_t N, float eps, int round_scale, int fp8_kind,
+                                void* stream);
 
 /* triton_silu_and_block_quant_forward, linghe/utils/silu.py:279-335.
  * x bf16 [M, 2n] (gate | up).  Outputs as fq_blockwise_quant with N = n. */

@@ -38,13 +38,13 @@ SIGNATURES = {
     "fq_rmsnorm_bwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _P],
     "fq_rmsnorm_bwd_noalloc": [_P, _P, _P, _P, _P, _P, _L, _L, _F, _P],
     "fq_rmsnorm_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _I, _I, _P],
-    "fq_rmsnorm_router_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _I, _P],
+    "fq_rmsnorm_router_quant_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _I, _P],
     "fq_swiglu_quant_fwd": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_swiglu_quant_bwd": [_P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_swiglu_quant_fwd": [_P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_swiglu_quant_bwd": [_P, _P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
 }
-OTHER_SYMBOLS = ["fq_version", "fq_last_error", "fq_rmsnorm_bwd_num_partials"]
+OTHER_SYMBOLS = ["fq_version", "fq_last_error", "fq_rmsnorm_bwd_num_partials", "fq_rmsnorm_router_scratch_bytes"]
 
 
 def _load() -> ctypes.CDLL:
@@ -63,6 +63,8 @@ def _load() -> ctypes.CDLL:
     lib.fq_last_error.restype = ctypes.c_char_p
     lib.fq_rmsnorm_bwd_num_partials.argtypes = [_L, _L]
     lib.fq_rmsnorm_bwd_num_partials.restype = _L
+    lib.fq_rmsnorm_router_scratch_bytes.argtypes = [_L, _L, _I]
+    lib.fq_rmsnorm_router_scratch_bytes.restype = _L
     return lib
 
 

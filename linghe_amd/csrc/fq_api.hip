@@ -273,24 +273,31 @@ int fq_swiglu_bwd(const void* g, const void* x, const void* weight, int weight_i
                       fn);
 }
 
-int fq_rmsnorm_router_quant_fwd(const void* x, const void* gamma, const void* route_weight, void* weight_scratch,
-                                void* y, float* rstd, float* logits, void* q, float* s, int64_t M, int64_t K,
-                                int64_t N, float eps, int round_scale, int fp8_kind, void* stream) {
+int64_t fq_rmsnorm_router_scratch_bytes(int64_t K, int64_t N, int weight_is_fp32) {
+  if (K <= 0 || N <= 0 || K > 8192 || N > 8192) return 0;
+  return fq::rmsnorm_router_scratch_bytes((int)K, (int)N, weight_is_fp32 != 0);
+}
+
+int fq_rmsnorm_router_quant_fwd(const void* x, const void* gamma, const void* route_weight, int weight_is_fp32,
+                                void* weight_scratch, void* y, float* rstd, float* logits, void* q, float* s,
+                                int64_t M, int64_t K, int64_t N, float eps, int round_scale, int fp8_kind,
+                                void* stream) {
   const char* fn = "fq_rmsnorm_router_quant_fwd";
   int rc = check_common(fn, M, K, round_scale, fp8_kind);
   if (rc) return rc;
   if ((rc = check_norm_shape(fn, M, K))) return rc;
   FQ_REQUIRE(M % 32 == 0, FQ_ERR_SHAPE, "%s: M (%lld) is not a multiple of 32", fn, (long long)M);
-  FQ_REQUIRE(N > 0 && N % 128 == 0 && N <= 512, FQ_ERR_SHAPE,
-             "%s: %lld router outputs (supported: 128, 256, 384, 512)", fn, (long long)N);
+  FQ_REQUIRE(N > 0 && N % 128 == 0 && N <= 8192, FQ_ERR_SHAPE,
+             "%s: %lld router outputs (supported: multiples of 128 up to 8192)", fn, (long long)N);
   if (M == 0) return FQ_OK;
   FQ_REQUIRE(x && gamma && route_weight && weight_scratch && y && rstd && logits && q && s, FQ_ERR_ARG,
              "%s: NULL pointer", fn);
   FQ_REQUIRE(aligned16(x) && aligned16(gamma) && aligned16(route_weight) && aligned16(weight_scratch) && aligned16(y),
              FQ_ERR_ARG, "%s: misaligned pointer", fn);
   FQ_REQUIRE((reinterpret_cast<uintptr_t>(q) & 7u) == 0, FQ_ERR_ARG, "%s: q must be 8-byte aligned", fn);
-  return check_launch(fq::launch_rmsnorm_router_quant(x, gamma, route_weight, weight_scratch, y, rstd, logits, q, s, M, (int)K, (int)N,
-                                                      eps, round_scale, fp8_kind, (hipStream_t)stream),
+  return check_launch(fq::launch_rmsnorm_router_quant(x, gamma, route_weight, weight_is_fp32 != 0, weight_scratch, y,
+                                                      rstd, logits, q, s, M, (int)K, (int)N, eps, round_scale,
+                                                      fp8_kind, (hipStream_t)stream),
                       fn);
 }
 

@@ -56,10 +56,13 @@ hipError_t launch_swiglu_rows_bwd(const void* g, const void* x, const void* weig
 hipError_t launch_block_quant(const void* x, void* q, float* s, int64_t M, int N, int round_scale, int kind,
                               hipStream_t stream);
 
-// RMSNorm + router GEMM (N <= 512 logits per row) + 1x128 quant; M a multiple of 32
-hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, void* wpacked, void* y,
-                                       float* rstd, float* logits, void* q, float* s, int64_t M, int K, int N,
-                                       float eps, int round_scale, int kind, hipStream_t stream);
+// RMSNorm + router GEMM + 1x128 quant; M a multiple of 32, N a multiple of 128, the router
+// weight bf16 or fp32; wpacked: rmsnorm_router_scratch_bytes() bytes
+int64_t rmsnorm_router_scratch_bytes(int K, int N, int weight_fp32);
+hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, int weight_fp32,
+                                       void* wpacked, void* y, float* rstd, float* logits, void* q, float* s,
+                                       int64_t M, int K, int N, float eps, int round_scale, int kind,
+                                       hipStream_t stream);
 
 // measurement aid: read read_bytes from src, write write_bytes to dst (both multiples of 16), no arithmetic
 hipError_t launch_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,

@@ -15,6 +15,13 @@
 // then the blocks) and takes any K; rmsnorm_router_quant_resident_kernel further
 // down keeps the rows in registers when they fit.
 //
+// An fp32 router weight (what Megatron keeps) is split the same way, W = hi + lo with
+// hi = bf16(W), lo = bf16(W - hi) (what is left is below 2^-17 |W|), and the two planes
+// are laid side by side as "virtual" columns 2n (hi) and 2n + 1 (lo): the GEMM runs on
+// 2N bf16 columns and the epilogue adds each pair, which sits in neighbouring lanes.
+// More than 512 virtual columns are cut into chunks of at most 512, one launch each;
+// only the first launch writes y, the codes, the scales and the statistic.
+//
 // One workgroup (4 or 8 waves) owns 32 rows and all N <= 512 logits of them and walks K
 // in blocks of 128 (one quantisation group per row):
 //   each thread normalises 2 rows x 8 columns of the block (16 lanes per row, so
@@ -81,31 +88,69 @@ __device__ __forceinline__ void router_rows_rstd(const uint16_t* rows, int n, fl
 // W [N, K] -> B operands in the order the main kernel reads them: one 16-byte piece
 // per (k block, 32-column tile, k step, lane), so that every B load of a wave is
 // 1 KB of contiguous memory.  (Read straight from the row-major matrix, each lane of
-// such a load would touch a cache line of its own.)
-__global__ __launch_bounds__(256) void pack_router_weight_kernel(const uint16_t* __restrict__ wr,
-                                                                 uint4* __restrict__ packed, int K, int N) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // piece number
-  const int64_t total = (int64_t)N * K / 8;
+// such a load would touch a cache line of its own.)  One launch packs the `vtiles`
+// 32-column tiles of one chunk, starting at virtual column vcol0; with an fp32 weight
+// virtual column v is plane v & 1 (0: bf16(W), 1: bf16 of the rest) of column v >> 1.
+template <bool FP32W>
+__global__ __launch_bounds__(256) void pack_router_weight_kernel(const void* __restrict__ wr,
+                                                                 uint4* __restrict__ packed, int K, int vcol0,
+                                                                 int vtiles) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // piece number inside the chunk
+  const int64_t total = (int64_t)vtiles * 32 * K / 8;
   if (idx >= total) return;
-  const int tiles = N / 32;
   const int lane = (int)(idx & 63);
   int64_t rest = idx >> 6;
   const int j = (int)(rest & 7);
   rest >>= 3;
-  const int tile = (int)(rest % tiles);
-  const int kb = (int)(rest / tiles);
-  const int n = tile * 32 + (lane & 31);
+  const int tile = (int)(rest % vtiles);
+  const int kb = (int)(rest / vtiles);
+  const int v = vcol0 + tile * 32 + (lane & 31);
   const int k = kb * kGroup + (lane >> 5) * 64 + j * 8;
-  packed[idx] = *(const uint4*)(wr + (int64_t)n * K + k);
+  if constexpr (!FP32W) {
+    packed[idx] = *(const uint4*)((const uint16_t*)wr + (int64_t)v * K + k);
+  } else {
+    const float4* src = (const float4*)((const float*)wr + (int64_t)(v >> 1) * K + k);
+    const float4 a = src[0], b = src[1];
+    float w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const uint4 hi = pack8_bf16(w);
+    if (v & 1) {
+      float back[8], lo[8];
+      unpack8(hi, back);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) lo[i] = w[i] - back[i];
+      packed[idx] = pack8_bf16(lo);
+    } else {
+      packed[idx] = hi;
+    }
+  }
+}
+
+// Where a launch puts its logits.  A chunk holds `real` columns of the [M, n_logits] matrix
+// starting at col0; with PAIR the accumulator columns come in (hi, lo) pairs in neighbouring
+// lanes and their sum is one real column.
+struct LogitsOut {
+  float* logits;
+  int n_logits;  // row stride
+  int col0;      // first real column of this launch
+};
+template <bool PAIR>
+__device__ __forceinline__ void store_logit(const LogitsOut& o, int64_t row, int vcol, float v) {
+  if constexpr (PAIR) {
+    v += dpp_mov<kDppQuadXor1>(v);  // lanes 2i, 2i+1 hold the two planes of one column
+    if ((vcol & 1) == 0) o.logits[row * o.n_logits + o.col0 + (vcol >> 1)] = v;
+  } else {
+    o.logits[row * o.n_logits + o.col0 + vcol] = v;
+  }
 }
 
 // WAVES waves per workgroup, TPW column tiles (of 32 logits) per wave: N = 32 * WAVES * TPW.
 // With 8 waves a thread owns one row x 8 columns of a k block, with 4 waves two rows.
-template <int KIND, bool ROUND, int TPW, int WAVES>
+// SIDE: this launch also writes y, the codes, the scales and the statistic (the first chunk does)
+template <int KIND, bool ROUND, int TPW, int WAVES, bool PAIR, bool SIDE>
 __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma, const uint4* __restrict__ wpacked,
-    uint16_t* __restrict__ y, float* __restrict__ rstd_out, float* __restrict__ logits, uint8_t* __restrict__ q,
-    float* __restrict__ s, int64_t M, int K, int N, float eps) {
+    uint16_t* __restrict__ y, float* __restrict__ rstd_out, LogitsOut lout, uint8_t* __restrict__ q,
+    float* __restrict__ s, int64_t M, int K, float eps) {
   __shared__ RouterShared sh;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -122,7 +167,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
     if (lane < 4) {
       const float mine = lane == 0 ? rs[0] : lane == 1 ? rs[1] : lane == 2 ? rs[2] : rs[3];
       sh.rstd[r + lane] = mine;
-      rstd_out[row0 + r + lane] = mine;
+      if constexpr (SIDE) rstd_out[row0 + r + lane] = mine;
     }
   }
   __syncthreads();
@@ -184,8 +229,6 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
         yv[i] = (a[i] * r) * g[i];
         m = fmaxf(m, fabsf(yv[i]));
       }
-      m = row16_max(m);
-      const float sc = make_scale<KIND, ROUND>(m);
       const uint4 hi = pack8_bf16(yv);
       float back[8], lo[8];
       unpack8(hi, back);
@@ -194,10 +237,14 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
       const int slot = ahalf * 32 + ((RPT * rg + u) ^ aj);
       sh.a[buf][0][aj][slot] = hi;
       sh.a[buf][1][aj][slot] = pack8_bf16(lo);
-      store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, hi);
-      const uint2 pk = quantize8<KIND, ROUND>(yv, make_quantum<ROUND>(sc));
-      store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
-      if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
+      if constexpr (SIDE) {
+        m = row16_max(m);
+        const float sc = make_scale<KIND, ROUND>(m);
+        store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, hi);
+        const uint2 pk = quantize8<KIND, ROUND>(yv, make_quantum<ROUND>(sc));
+        store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
+        if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
+      }
     }
     __syncthreads();
 #pragma unroll
@@ -242,7 +289,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int row = (v / 4) * 8 + half * 4 + (v % 4);
-      logits[(row0 + row) * N + col] = acc[t][v];
+      store_logit<PAIR>(lout, row0 + row, col, acc[t][v]);
     }
   }
 }
@@ -261,11 +308,11 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
 //     the MFMAs so that the memory pipeline and the matrix cores work together;
 //   sweep 2, from registers: logits *= rstd; y = (x*rstd)*gamma -> bf16, codes and
 //     scales, streamed out.
-template <int KIND, bool ROUND, int TPW, int WAVES, int KB, int WDEPTH>
+template <int KIND, bool ROUND, int TPW, int WAVES, int KB, int WDEPTH, bool PAIR>
 __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma, const uint4* __restrict__ wpacked,
-    uint16_t* __restrict__ y, float* __restrict__ rstd_out, float* __restrict__ logits, uint8_t* __restrict__ q,
-    float* __restrict__ s, int64_t M, int K, int N, float eps) {
+    uint16_t* __restrict__ y, float* __restrict__ rstd_out, LogitsOut lout, uint8_t* __restrict__ q,
+    float* __restrict__ s, int64_t M, int K, float eps) {
   __shared__ RouterShared sh;
   __shared__ uint4 sgamma[KB * 16];  // gamma, 8 columns per piece
   const int lane = threadIdx.x & 63;
@@ -384,7 +431,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int row = (v / 4) * 8 + half * 4 + (v % 4);
-      logits[(row0 + row) * N + col] = acc[t][v] * sh.rstd[row];
+      store_logit<PAIR>(lout, row0 + row, col, acc[t][v] * sh.rstd[row]);
     }
   }
 
@@ -417,55 +464,85 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
   }
 }
 
-hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, void* wpacked, void* y,
-                                       float* rstd, float* logits, void* q, float* s, int64_t M, int K, int N,
-                                       float eps, int round_scale, int kind, hipStream_t stream) {
+int64_t rmsnorm_router_scratch_bytes(int K, int N, int weight_fp32) {
+  return (int64_t)N * K * (weight_fp32 ? 4 : 2);  // the bf16 planes of W in operand order
+}
+
+hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, int weight_fp32,
+                                       void* wpacked, void* y, float* rstd, float* logits, void* q, float* s,
+                                       int64_t M, int K, int N, float eps, int round_scale, int kind,
+                                       hipStream_t stream) {
   if (M == 0) return hipSuccess;
-  {
-    const int64_t pieces = (int64_t)N * K / 8;
-    hipLaunchKernelGGL(pack_router_weight_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, stream,
-                       (const uint16_t*)wr, (uint4*)wpacked, K, N);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-  }
+  const int vcols = weight_fp32 ? 2 * N : N;  // virtual bf16 columns
   const dim3 grid((unsigned)(M / kRouterRows));
-  const int tiles = N / 32;
-  // 8 waves when the column tiles split evenly over them (N = 256, 512), else 4;
-  // rows held in registers when they fit beside the operands and K is one of the
-  // instantiated widths: one column tile per wave (N = 128, 256), K = 1024 or 2048;
-  // streamed twice otherwise
 #define FQ_ROUTER_ARGS(WAVESV)                                                                                  \
-  grid, dim3(64 * WAVESV), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)wpacked,        \
-      (uint16_t*)y, rstd, logits, (uint8_t*)q, s, M, K, N, eps
+  grid, dim3(64 * WAVESV), 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, (const uint4*)chunk_w,        \
+      (uint16_t*)y, rstd, lout, (uint8_t*)q, s, M, K, eps
 #define FQ_ROUTER_STREAMED(KINDV, ROUNDV, TPWV, WAVESV)                                                         \
-  hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, TPWV, WAVESV>), FQ_ROUTER_ARGS(WAVESV))
-#define FQ_ROUTER_RESIDENT(KINDV, ROUNDV, TPWV, WAVESV)                                                         \
-  if (K == 2048)                                                                                                \
-    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, 16, 2>),              \
-                       FQ_ROUTER_ARGS(WAVESV));                                                                 \
-  else if (K == 1024)                                                                                           \
-    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, 8, 2>),               \
+  if (first)                                                                                                    \
+    hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, TPWV, WAVESV, PAIRV, true>),                 \
                        FQ_ROUTER_ARGS(WAVESV));                                                                 \
   else                                                                                                          \
-    FQ_ROUTER_STREAMED(KINDV, ROUNDV, TPWV, WAVESV)
+    hipLaunchKernelGGL((rmsnorm_router_quant_kernel<KINDV, ROUNDV, TPWV, WAVESV, PAIRV, false>),                \
+                       FQ_ROUTER_ARGS(WAVESV))
+#define FQ_ROUTER_RESIDENT(KINDV, ROUNDV, TPWV, WAVESV)                                                         \
+  if (single && K == 2048)                                                                                      \
+    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, 16, 2, PAIRV>),       \
+                       FQ_ROUTER_ARGS(WAVESV));                                                                 \
+  else if (single && K == 1024)                                                                                 \
+    hipLaunchKernelGGL((rmsnorm_router_quant_resident_kernel<KINDV, ROUNDV, TPWV, WAVESV, 8, 2, PAIRV>),        \
+                       FQ_ROUTER_ARGS(WAVESV));                                                                 \
+  else {                                                                                                        \
+    FQ_ROUTER_STREAMED(KINDV, ROUNDV, TPWV, WAVESV);                                                            \
+  }
 #define FQ_ROUTER_KIND(GO, TPWV, WAVESV)                                                                        \
   if (kind == kE5M2) {                                                                                          \
     if (round_scale) { GO(kE5M2, true, TPWV, WAVESV); } else { GO(kE5M2, false, TPWV, WAVESV); }                \
   } else {                                                                                                      \
     if (round_scale) { GO(kE4M3, true, TPWV, WAVESV); } else { GO(kE4M3, false, TPWV, WAVESV); }                \
   }
-  switch (tiles) {
-    case 4: FQ_ROUTER_KIND(FQ_ROUTER_RESIDENT, 1, 4) break;
-    case 8: FQ_ROUTER_KIND(FQ_ROUTER_RESIDENT, 1, 8) break;
-    case 12: FQ_ROUTER_KIND(FQ_ROUTER_STREAMED, 3, 4) break;
-    case 16: FQ_ROUTER_KIND(FQ_ROUTER_STREAMED, 2, 8) break;
-    default: return hipErrorInvalidValue;
+  // 8 waves when the column tiles split evenly over them (256, 512 virtual columns), else 4;
+  // rows held in registers when there is one chunk, one column tile per wave (128 or 256
+  // virtual columns) and K is one of the instantiated widths (1024, 2048); streamed twice
+  // otherwise
+#define FQ_ROUTER_TILES()                                                   \
+  switch (vtiles) {                                                         \
+    case 4: FQ_ROUTER_KIND(FQ_ROUTER_RESIDENT, 1, 4) break;                 \
+    case 8: FQ_ROUTER_KIND(FQ_ROUTER_RESIDENT, 1, 8) break;                 \
+    case 12: FQ_ROUTER_KIND(FQ_ROUTER_STREAMED, 3, 4) break;                \
+    case 16: FQ_ROUTER_KIND(FQ_ROUTER_STREAMED, 2, 8) break;                \
+    default: return hipErrorInvalidValue;                                   \
   }
+  const bool single = vcols <= 512;
+  for (int v0 = 0; v0 < vcols; v0 += 512) {
+    const int vtiles = (vcols - v0 < 512 ? vcols - v0 : 512) / 32;
+    const bool first = v0 == 0;
+    uint4* chunk_w = (uint4*)wpacked + (int64_t)v0 * K / 8;
+    const int64_t pieces = (int64_t)vtiles * 32 * K / 8;
+    const dim3 pgrid((unsigned)((pieces + 255) / 256));
+    if (weight_fp32)
+      hipLaunchKernelGGL(pack_router_weight_kernel<true>, pgrid, dim3(256), 0, stream, wr, chunk_w, K, v0, vtiles);
+    else
+      hipLaunchKernelGGL(pack_router_weight_kernel<false>, pgrid, dim3(256), 0, stream, wr, chunk_w, K, v0, vtiles);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const LogitsOut lout{logits, N, weight_fp32 ? v0 / 2 : v0};
+    if (weight_fp32) {
+      constexpr bool PAIRV = true;
+      FQ_ROUTER_TILES()
+    } else {
+      constexpr bool PAIRV = false;
+      FQ_ROUTER_TILES()
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+#undef FQ_ROUTER_TILES
 #undef FQ_ROUTER_KIND
 #undef FQ_ROUTER_RESIDENT
 #undef FQ_ROUTER_STREAMED
 #undef FQ_ROUTER_ARGS
-  return hipGetLastError();
+  return hipSuccess;
 }
 
 }  // namespace fq

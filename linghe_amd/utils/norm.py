@@ -170,7 +170,7 @@ def triton_rms_norm_fp32_gemm_block_quant_forward(
     Args:
         x: input tensor, bf16 [M, K]
         norm weight: weight tensor of rms norm, bf16 [K]
-        route_weight: moe router weight, bf16 [N, K], N in {128, 256, 384, 512}
+        route_weight: moe router weight [N, K], bf16 or fp32, N a multiple of 128
         eps: epsilon of rms norm
         output_mode: 0 or 1
             0: only output non-transpose quantizatino tensor (and y, rms, logits)
@@ -208,11 +208,16 @@ def triton_rms_norm_fp32_gemm_block_quant_forward(
         return y, rms, logits, x_q, x_s, xt_q, xt_s
     with _lib.on_device(device):
         if output_mode == 0:
-            _lib.require_device_bf16(route_weight, "route_weight")
-            assert N <= 512, f"{N=} router outputs: at most 512 are supported"
-            scratch = torch.empty_like(route_weight)  # route_weight re-ordered for the matrix cores
+            if route_weight.dtype not in (torch.bfloat16, torch.float32):
+                raise TypeError(f"route_weight must be bfloat16 or float32, got {route_weight.dtype}")
+            if not route_weight.is_cuda:
+                raise RuntimeError("route_weight must live on the GPU: the HIP kernels are the only implementation")
+            w_fp32 = int(route_weight.dtype == torch.float32)
+            # route_weight re-ordered for the matrix cores (an fp32 weight as two bf16 planes)
+            scratch = torch.empty(int(_lib.lib.fq_rmsnorm_router_scratch_bytes(K, N, w_fp32)), dtype=torch.uint8,
+                                  device=device)
             _lib.check(_lib.lib.fq_rmsnorm_router_quant_fwd(
-                _lib.ptr(x), _lib.ptr(norm_weight), _lib.ptr(route_weight), _lib.ptr(scratch), _lib.ptr(y), _lib.ptr(rms),
+                _lib.ptr(x), _lib.ptr(norm_weight), _lib.ptr(route_weight), w_fp32, _lib.ptr(scratch), _lib.ptr(y), _lib.ptr(rms),
                 _lib.ptr(logits), _lib.ptr(x_q), _lib.ptr(x_s), M, K, N, float(eps), int(bool(round_scale)),
                 _lib.FQ_E4M3, _lib.stream_of(x)))
         else:

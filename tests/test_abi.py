@@ -81,13 +81,15 @@ def test_c_side_validation_without_gpu():
     # 128x128 block quant needs whole blocks of rows
     rc = L.fq_block_quant(None, None, None, 100, 256, 0, 0, None)
     assert rc == -2 and b"128" in L.fq_last_error()
-    # router GEMM: at most 512 outputs, rows in groups of 32
-    rc = L.fq_rmsnorm_router_quant_fwd(None, None, None, None, None, None, None, None, None, 128, 2048, 640, 1e-6, 0, 0,
-                                       None)
+    # router GEMM: outputs in multiples of 128, rows in groups of 32
+    rc = L.fq_rmsnorm_router_quant_fwd(None, None, None, 0, None, None, None, None, None, None, 128, 2048, 200, 1e-6,
+                                       0, 0, None)
     assert rc == -2 and b"router" in L.fq_last_error()
-    rc = L.fq_rmsnorm_router_quant_fwd(None, None, None, None, None, None, None, None, None, 100, 2048, 256, 1e-6, 0, 0,
-                                       None)
+    rc = L.fq_rmsnorm_router_quant_fwd(None, None, None, 1, None, None, None, None, None, None, 100, 2048, 256, 1e-6,
+                                       0, 0, None)
     assert rc == -2
+    assert L.fq_rmsnorm_router_scratch_bytes(2048, 256, 0) == 256 * 2048 * 2
+    assert L.fq_rmsnorm_router_scratch_bytes(2048, 256, 1) == 256 * 2048 * 4
     # gather + pad: the output row count is a sum of multiples of 16; probs and prob_out go together
     rc = L.fq_batched_pad_permute_quant(None, None, 0, 4, 1, None, None, 0, None, None, None, None, None, 64, 100, 256,
                                         0, 0, None)

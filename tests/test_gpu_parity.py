@@ -396,18 +396,27 @@ def test_block_quant(gpu, M, N, round_scale):
 
 
 # ------------------------------------------------------------------ RMSNorm + router GEMM + quant
-@pytest.mark.parametrize("M,N,K", [(8192, 256, 2048), (256, 128, 1536), (128, 512, 4096), (384, 384, 7168),
-                                   (256, 128, 1024), (128, 256, 1024), (128, 128, 2048)])
+@pytest.mark.parametrize("M,N,K,wdtype", [
+    (8192, 256, 2048, torch.bfloat16), (256, 128, 1536, torch.bfloat16), (128, 512, 4096, torch.bfloat16),
+    (384, 384, 7168, torch.bfloat16), (256, 128, 1024, torch.bfloat16), (128, 256, 1024, torch.bfloat16),
+    (128, 128, 2048, torch.bfloat16),
+    # an fp32 router weight (what Megatron keeps), as two bf16 planes: register-resident (2N = 256) and streamed forms
+    (8192, 256, 2048, torch.float32), (256, 128, 2048, torch.float32), (128, 128, 1024, torch.float32),
+    (256, 256, 1536, torch.float32),
+    # more than 512 (virtual) columns: one launch per chunk of 512
+    (256, 1024, 2048, torch.bfloat16), (128, 640, 1536, torch.bfloat16), (128, 384, 2048, torch.float32),
+    (128, 1024, 1024, torch.float32)])
 @pytest.mark.parametrize("round_scale", [False, True])
-def test_rms_norm_fp32_gemm_block_quant(gpu, M, N, K, round_scale):
-    """reference tests/test_norm.py:251-287 (x = randn**2, weights randn)."""
+def test_rms_norm_fp32_gemm_block_quant(gpu, M, N, K, wdtype, round_scale):
+    """reference tests/test_norm.py:251-287 (x = randn**2, weights randn; the reference's
+    router weight is whatever dtype the caller holds, loaded .to(float32))."""
     from linghe_amd.utils.norm import triton_rms_norm_fp32_gemm_block_quant_forward as fn
 
-    announce("rmsnorm + router gemm + quant", M, N, K, round_scale)
+    announce("rmsnorm + router gemm + quant", M, N, K, wdtype, round_scale)
     g = gen(24)
     x = (torch.randn(M, K, generator=g) ** 2).to(torch.bfloat16)
     nw = torch.randn(K, generator=g).to(torch.bfloat16)
-    rw = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    rw = torch.randn(N, K, generator=g).to(wdtype)
     xd, nwd, rwd = _dev(x, gpu), _dev(nw, gpu), _dev(rw, gpu)
     y, rms, logits, q, s, qt0, st0 = fn(xd, nwd, rwd, round_scale=round_scale, output_mode=0)
     torch.cuda.synchronize()
@@ -420,10 +429,15 @@ def test_rms_norm_fp32_gemm_block_quant(gpu, M, N, K, round_scale):
     pin = O.rms_gemm_block_quant_forward(x, nw, rw, round_scale=round_scale, rstd=rms.cpu())
     assert torch.equal(pin[0].view(torch.int16), y.cpu().view(torch.int16))
     check_quant_pair("router.row", pin[3], pin[4], q, s, **EXACT)
-    # logits: fp32 GEMM accuracy (the two-term bf16 split leaves < 2^-17 of each |y|;
-    # the reference's own check allows rtol 1e-3, atol 0.1)
-    scale = float((pin[0].float().abs() @ rw.float().abs().t()).max())
-    err = float((logits.cpu() - pin[2]).abs().max())
+    # logits: fp32 GEMM accuracy (the two-term bf16 splits leave < 2^-17 of each |y| and of
+    # each |w| of an fp32 weight; the reference's own check allows rtol 1e-3, atol 0.1).
+    # Judged against the fp64 product of the fp32 y the oracle forms.
+    y32 = (x.float() * rms.cpu()[:, None]) * nw.float()
+    exact = y32.double() @ rw.double().t()
+    scale = float((y32.abs().double() @ rw.double().abs().t()).max())
+    err = float((logits.cpu().double() - exact).abs().max())
+    err_oracle = float((pin[2].double() - exact).abs().max())
+    print(f"[parity] router.logits vs fp64: kernel {err:.3e}, torch fp32 matmul {err_oracle:.3e}", flush=True)
     print(f"[parity] router.logits: max abs err {err:.3e}, sum|y||w| max {scale:.3e}", flush=True)
     assert err <= 2e-5 * scale
     torch.testing.assert_close(logits.cpu(), ref[2], rtol=1e-3, atol=0.1)
