@@ -31,6 +31,7 @@ namespace fq {
 #ifndef FQ_ROW_LDNT
 #define FQ_ROW_LDNT 1
 #endif
+
 __device__ __forceinline__ void st16(void* p, const uint4& v) { store16<FQ_NT_ROWS != 0>(p, v); }
 __device__ __forceinline__ void st8(void* p, const uint2& v) { store8<FQ_NT_ROWS != 0>(p, v); }
 __device__ __forceinline__ uint4 ld16(const void* p) { return load16<FQ_ROW_LDNT != 0>(p); }
@@ -259,8 +260,24 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
                                                         int64_t M, int n, float eps, int rows_per_wg) {
   __shared__ RowShared<T> sh;
   const int tid = threadIdx.x;
-  uint4 gm[NCHUNK];
-  load_row<T, NCHUNK>(gamma, n, gm);
+  const int chunks = n >> 3;
+  // A thread's chunk k is column chunk tid + k*T.  Beyond the end of the row it reads the
+  // row's last chunk again (a valid address, no branch) and takes part with gamma = 0:
+  // its share of the row sums is zero and none of its results is stored.
+  int cidx[NCHUNK];
+  bool live[NCHUNK];
+  float w[NCHUNK][8];  // gamma, unpacked once
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) {
+    const int c = tid + k * T;
+    live[k] = c < chunks;
+    cidx[k] = live[k] ? c : chunks - 1;
+    unpack8(*(const uint4*)(gamma + cidx[k] * 8), w[k]);
+    if (!live[k]) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) w[k][j] = 0.f;
+    }
+  }
   float acc[NCHUNK][8];
 #pragma unroll
   for (int k = 0; k < NCHUNK; ++k)
@@ -270,22 +287,33 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
   // rows blockIdx.x, blockIdx.x + G, blockIdx.x + 2G, ...: at any moment the
   // workgroups of the grid work on neighbouring rows (one moving front in memory)
   const int64_t G = gridDim.x;
-  const int64_t r0 = blockIdx.x;
-  const int64_t r1 = M;
   (void)rows_per_wg;
 
-  auto process = [&](uint4 (&rx)[NCHUNK], uint4 (&rg)[NCHUNK], int64_t row, int parity) {
+  // One row in registers at a time (about 100 of them with two chunks per thread), so
+  // that two 512-thread workgroups fit a CU and cover each other's waits.  Prefetching
+  // the next row's packed data into a second register set spills (142 -> 198 us at
+  // 16384 x 7168 with 512 threads, 155 -> 179 us with 256 threads and four chunks).
+  int parity = 0;
+  for (int64_t row = blockIdx.x; row < M; row += G) {
+    uint4 rx[NCHUNK], rg[NCHUNK];
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) {
+      rx[k] = load16<FQ_ROW_LDNT != 0>(x + row * n + cidx[k] * 8);
+      rg[k] = load16<FQ_ROW_LDNT != 0>(dy + row * n + cidx[k] * 8);
+    }
     double ss = 0.0;
-    if constexpr (!REUSE) ss = sumsq<NCHUNK>(rx);
     float dot = 0.f;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
-      float a[8], g[8], w[8];
+      float a[8], g[8];
       unpack8(rx[k], a);
       unpack8(rg[k], g);
-      unpack8(gm[k], w);
+      if constexpr (!REUSE) {
+        const float part = sumsq8(rx[k]);
+        ss += (double)(live[k] ? part : 0.f);
+      }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
+      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[k][j], dot);
     }
     if constexpr (REUSE) {
       float unused = 0.f;
@@ -293,6 +321,7 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
     } else {
       block_sum2<T>(ss, dot, sh, parity);
     }
+    parity ^= 1;
     forget<NCHUNK>(rx);
     forget<NCHUNK>(rg);
     float r;
@@ -301,32 +330,15 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
     const float coef = ((r * r) * r) * dot / (float)n;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
-      const int c = tid + k * T;
-      float a[8], g[8], w[8], o[8];
+      float a[8], g[8], o[8];
       unpack8(rx[k], a);
       unpack8(rg[k], g);
-      unpack8(gm[k], w);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        o[j] = (r * g[j]) * w[j] - coef * a[j];
-        acc[k][j] += (a[j] * g[j]) * r;
+        o[j] = (r * g[j]) * w[k][j] - coef * a[j];
+        acc[k][j] = __builtin_fmaf(a[j] * g[j], r, acc[k][j]);  // dgamma: one rounding fewer per term
       }
-      if (c * 8 < n) st16(dx + row * n + c * 8, pack8_bf16(o));
-    }
-  };
-
-  // One row in registers at a time (about 100 of them with two chunks per thread), so
-  // that two 512-thread workgroups fit a CU and cover each other's waits.  Prefetching
-  // the next row into a second register set costs that second workgroup and is slower
-  // (179 vs 155 us at 16384 x 7168).
-  {
-    uint4 xa[NCHUNK], ga[NCHUNK];
-    int parity = 0;
-    for (int64_t row = r0; row < r1; row += G) {
-      load_row<T, NCHUNK, FQ_ROW_LDNT != 0>(x + row * n, n, xa);
-      load_row<T, NCHUNK, FQ_ROW_LDNT != 0>(dy + row * n, n, ga);
-      process(xa, ga, row, parity);
-      parity ^= 1;
+      if (live[k]) st16(dx + row * n + cidx[k] * 8, pack8_bf16(o));
     }
   }
   // every workgroup writes its (possibly zero) partial: the reduction reads all of them
