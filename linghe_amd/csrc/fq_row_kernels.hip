@@ -97,6 +97,21 @@ __device__ __forceinline__ void load_row(const uint16_t* row, int n, uint4 (&raw
   }
 }
 
+// The same without a branch: a chunk beyond the end of the row reads the row's last
+// chunk again (a valid address).  Loads that sit behind a per-lane condition are issued
+// one by one, each behind its own exec-mask branch; these go out back to back.  What is
+// computed from such a chunk must not be stored, and must be left out of row sums
+// (sumsq_live).
+template <int T, int NCHUNK, bool STREAM = false>
+__device__ __forceinline__ void load_row_clamped(const uint16_t* row, int n, uint4 (&raw)[NCHUNK]) {
+  const int last = (n >> 3) - 1;
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) {
+    const int c = threadIdx.x + k * T;
+    raw[k] = load16<STREAM>(row + (c < last ? c : last) * 8);
+  }
+}
+
 // make the compiler forget what it knows about a packed row, so that the fp32
 // copies made before a reduction are not kept alive across it (they are cheap to
 // remake and cost four times the registers)
@@ -124,6 +139,17 @@ __device__ __forceinline__ double sumsq(const uint4 (&raw)[NCHUNK]) {
   double ss = 0.0;
 #pragma unroll
   for (int k = 0; k < NCHUNK; ++k) ss += (double)sumsq8(raw[k]);
+  return ss;
+}
+// the same for a row fetched by load_row_clamped: chunks beyond the end of the row count as zero
+template <int T, int NCHUNK>
+__device__ __forceinline__ double sumsq_live(const uint4 (&raw)[NCHUNK], int n) {
+  double ss = 0.0;
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) {
+    const float part = sumsq8(raw[k]);
+    ss += (double)((((int)threadIdx.x & (T - 1)) + k * T) * 8 < n ? part : 0.f);  // T a power of two; a wave-per-row kernel passes T = 64
+  }
   return ss;
 }
 
@@ -159,7 +185,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
     if constexpr (REUSE) {
       r = rstd[row];
     } else {
-      double ss = sumsq<NCHUNK>(raw);
+      double ss = sumsq_live<T, NCHUNK>(raw, n);
       float dummy = 0.f;
       block_sum2<T>(ss, dummy, sh, parity);
       r = rstd_from_sumsq((float)ss, n, eps);
@@ -196,19 +222,19 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
     uint4 buf[NCHUNK];
     int parity = 0;
     for (int64_t row = r0; row < r1; row += G) {
-      load_row<T, NCHUNK, FQ_ROW_LDNT != 0>(x + row * n, n, buf);
+      load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + row * n, n, buf);
       process(buf, row, parity);
       parity ^= 1;
     }
     return;
   }
   uint4 bufA[NCHUNK], bufB[NCHUNK];
-  load_row<T, NCHUNK, FQ_ROW_LDNT != 0>(x + r0 * n, n, bufA);
+  load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + r0 * n, n, bufA);
   for (int64_t row = r0; row < r1; row += 2 * G) {
-    if (row + G < r1) load_row<T, NCHUNK, FQ_ROW_LDNT != 0>(x + (row + G) * n, n, bufB);
+    if (row + G < r1) load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + (row + G) * n, n, bufB);
     process(bufA, row, 0);
     if (row + G < r1) {
-      if (row + 2 * G < r1) load_row<T, NCHUNK, FQ_ROW_LDNT != 0>(x + (row + 2 * G) * n, n, bufA);
+      if (row + 2 * G < r1) load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + (row + 2 * G) * n, n, bufA);
       process(bufB, row + G, 1);
     }
   }
@@ -220,6 +246,10 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
 // CU holds its 32 waves and a 16384-row input is two rows per wave with no tail.
 // Same arithmetic as everywhere else: 8-element group sums added in double.
 // ---------------------------------------------------------------------------
+// U: 16-byte loads per lane and step (a step covers U * 512 columns); 4 for rows of at most 2048
+// columns, 8 beyond.  The loads carry no per-lane condition: a chunk beyond the end of the row
+// reads the row's last chunk again and counts as zero.
+template <int U>
 __global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict__ x, float* __restrict__ rstd,
                                                      int64_t M, int n, float eps) {
   const int lane = threadIdx.x;
@@ -232,16 +262,18 @@ __global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict_
     const int64_t row = M - 1 - k;
     const uint4* p = (const uint4*)(x + row * n);
     double ss = 0.0;
-    for (int c0 = 0; c0 < chunks; c0 += 512) {
-      uint4 v[8];
+    for (int c0 = 0; c0 < chunks; c0 += U * 64) {
+      uint4 v[U];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < U; ++u) {
         const int c = c0 + u * 64 + lane;
-        v[u] = make_uint4(0, 0, 0, 0);
-        if (c < chunks) v[u] = p[c];
+        v[u] = p[c < chunks ? c : chunks - 1];
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u) ss += (double)sumsq8(v[u]);
+      for (int u = 0; u < U; ++u) {
+        const float part = sumsq8(v[u]);
+        ss += (double)(c0 + u * 64 + lane < chunks ? part : 0.f);
+      }
     }
     ss = wave_sum_d(ss);
     if (lane == 0) rstd[row] = rstd_from_sumsq((float)ss, n, eps);
@@ -370,12 +402,13 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_wave_kernel(const uint16_t* _
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int chunks = n >> 3;
-  uint4 gm[NCHUNK];
+  float w[NCHUNK][8];  // gamma, unpacked once; zero beyond the end of the row
 #pragma unroll
   for (int k = 0; k < NCHUNK; ++k) {
     const int c = lane + k * 64;
-    gm[k] = make_uint4(0, 0, 0, 0);
-    if (c < chunks) gm[k] = *(const uint4*)(gamma + c * 8);
+    uint4 gm = make_uint4(0, 0, 0, 0);
+    if (c < chunks) gm = *(const uint4*)(gamma + c * 8);
+    unpack8(gm, w[k]);
   }
   float acc[NCHUNK][8];
 #pragma unroll
@@ -388,43 +421,40 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_wave_kernel(const uint16_t* _
     uint4 rx[NCHUNK], rg[NCHUNK];
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
+      // no per-lane condition on the loads: a chunk beyond the end of the row reads the last
+      // chunk again; its gamma is zero, so it adds nothing to the row sums, and it is not stored
       const int c = lane + k * 64;
-      rx[k] = make_uint4(0, 0, 0, 0);
-      rg[k] = make_uint4(0, 0, 0, 0);
-      if (c < chunks) {
-        rx[k] = ld16(x + row * n + c * 8);
-        rg[k] = ld16(dy + row * n + c * 8);
-      }
+      const int cc = c < chunks ? c : chunks - 1;
+      rx[k] = ld16(x + row * n + cc * 8);
+      rg[k] = ld16(dy + row * n + cc * 8);
     }
     float dot = 0.f;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
-      float a[8], g[8], w[8];
+      float a[8], g[8];
       unpack8(rx[k], a);
       unpack8(rg[k], g);
-      unpack8(gm[k], w);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[j], dot);
+      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(a[j] * g[j], w[k][j], dot);
     }
     dot = wave_sum(dot);
     float r;
     if constexpr (REUSE) {
       r = rstd_in[row];
     } else {
-      r = rstd_from_sumsq((float)wave_sum_d(sumsq<NCHUNK>(rx)), n, eps);
+      r = rstd_from_sumsq((float)wave_sum_d(sumsq_live<64, NCHUNK>(rx, n)), n, eps);
     }
     const float coef = ((r * r) * r) * dot / (float)n;
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
       const int c = lane + k * 64;
-      float a[8], g[8], w[8], o[8];
+      float a[8], g[8], o[8];
       unpack8(rx[k], a);
       unpack8(rg[k], g);
-      unpack8(gm[k], w);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        o[j] = (r * g[j]) * w[j] - coef * a[j];
-        acc[k][j] += (a[j] * g[j]) * r;
+        o[j] = (r * g[j]) * w[k][j] - coef * a[j];
+        acc[k][j] = __builtin_fmaf(a[j] * g[j], r, acc[k][j]);
       }
       if (c < chunks) st16(dx + row * n + c * 8, pack8_bf16(o));
     }
@@ -558,7 +588,8 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
                                    scale, rstd, M, n, eps, rows_per_wg);)
   // quant: 0 = bf16 output, 1 = fp8 codes + scales, 2 = statistic only (its own kernel)
   if (quant == 2) {
-    hipLaunchKernelGGL(rowstat_kernel, grid, dim3(64), 0, stream, (const uint16_t*)x, rstd, M, n, eps);
+    if (n <= 2048) hipLaunchKernelGGL(rowstat_kernel<4>, grid, dim3(64), 0, stream, (const uint16_t*)x, rstd, M, n, eps);
+    else hipLaunchKernelGGL(rowstat_kernel<8>, grid, dim3(64), 0, stream, (const uint16_t*)x, rstd, M, n, eps);
   } else if (!quant) {
     if (reuse_rstd) { FQ_LAUNCH_FWD(true, 0, kE4M3, false) } else { FQ_LAUNCH_FWD(false, 0, kE4M3, false) }
   } else if (n > 2048) {
@@ -724,13 +755,11 @@ __global__ __launch_bounds__(64) void swiglu_fwd_rows_kernel(const uint16_t* __r
       uint4 r1[4], r2[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
+        // unconditional loads: beyond the end of the row the last chunk is read again (never stored)
         const int c = c0 + u * 64 + lane;
-        r1[u] = make_uint4(0, 0, 0, 0);
-        r2[u] = make_uint4(0, 0, 0, 0);
-        if (c < chunks) {
-          r1[u] = ld16(p + c * 8);
-          r2[u] = ld16(p + n + c * 8);
-        }
+        const int cc = c < chunks ? c : chunks - 1;
+        r1[u] = ld16(p + cc * 8);
+        r2[u] = ld16(p + n + cc * 8);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
