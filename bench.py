@@ -358,6 +358,60 @@ def build_cases(names, dev):
 
     add("next_block_quant", build=block_quant_case)
 
+    # ---------------------------------------------------------------- the quantisers with no fused pre-op
+    def plain_quant_case(name):
+        g = torch.Generator().manual_seed(1105)
+        if name == "a8_batch_blockwise":  # the activations of cfg3's experts: 65536 x 512, same Zipf counts
+            d = lazy.setdefault("cfg3", configs.cfg3_batched_swiglu())
+            counts = d["counts"]
+            M, N = sum(counts), 512
+        else:
+            counts = None
+            M, N = 8192, 2048
+        x_cpu = torch.randn(M, N, generator=g).to(torch.bfloat16)
+        blocks = sum((c + 127) // 128 for c in counts) if counts else (M + 127) // 128
+        cnt = torch.tensor(counts, dtype=torch.int32, device=dev) if counts else None
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), q=torch.empty((M, N), device=dev, dtype=FP8),
+                     s=torch.empty((M * (N // 128),), device=dev, dtype=torch.float32))
+            if name != "a8_group":
+                s["qt"] = torch.empty((M * N,), device=dev, dtype=FP8)
+                s["st"] = torch.empty((blocks * N,), device=dev, dtype=torch.float32)
+            if name == "a8_blockwise":
+                s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, N, 0, 2, _lib.FQ_E4M3,
+                             stream)
+            elif name == "a8_group":
+                s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), M, N, 0, _lib.FQ_E4M3, stream)
+            else:
+                s["args"] = (_p(s["x"]), _p(cnt), 0, len(counts), blocks, _p(s["q"]), _p(s["s"]), _p(s["qt"]),
+                             _p(s["st"]), M, N, 0, _lib.FQ_E4M3, stream)
+            return s
+
+        fn = {"a8_blockwise": L.fq_blockwise_quant, "a8_group": L.fq_group_quant,
+              "a8_batch_blockwise": L.fq_batched_blockwise_quant}[name]
+
+        def launch(s):
+            _lib.check(fn(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            if name == "a8_blockwise":
+                return O.blockwise_quant(x_cpu, False)
+            if name == "a8_group":
+                return O.group_quant_1x128(x_cpu, False)
+            return O.batch_blockwise_quant(x_cpu, counts, False)
+
+        row = M * N + 4 * M * (N // 128)
+        col = M * N + 4 * blocks * N
+        entry = {"a8_blockwise": "triton_blockwise_quant(output_mode=2)", "a8_group": "triton_group_quant",
+                 "a8_batch_blockwise": "triton_batch_blockwise_quant"}[name]
+        return Case(name, entry, [M, N], (2 * M * N, row + (0 if name == "a8_group" else col)), make_set, launch,
+                    cpu_fn)
+
+    for _n in ("a8_blockwise", "a8_group", "a8_batch_blockwise"):
+        add(_n, build=lambda _n=_n: plain_quant_case(_n))
+
     # ---------------------------------------------------------------- next row: RMSNorm + router GEMM + quant
     def router_case():
         M, N, K = 8192, 256, 2048
@@ -511,7 +565,7 @@ def load_traffic_table():
 
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
-       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2",
+       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "a8_blockwise", "a8_group", "a8_batch_blockwise",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router",
        "stream_read", "stream_copy"]
 
