@@ -124,6 +124,34 @@ def build_cases(names, dev):
     add("cfg1_pow2", build=lambda: rms_quant_case("cfg1_pow2", configs.cfg1_rmsnorm_quant(), 2, True))
     add("cfg5b", build=lambda: rms_quant_case("cfg5b", cfg5(), 2))
     add("cfg5c", build=lambda: rms_quant_case("cfg5c", cfg5(), 1))
+    # output_mode 0 (row-wise codes only: the first forward of a layer that will be recomputed)
+    add("cfg1_mode0", build=lambda: rms_quant_case("cfg1_mode0", configs.cfg1_rmsnorm_quant(), 0))
+    add("cfg5_mode0", build=lambda: rms_quant_case("cfg5_mode0", cfg5(), 0))
+
+    # ---------------------------------------------------------------- bf16 RMSNorm forward (a2)
+    def rms_fwd_case():
+        d = cfg5()
+        x_cpu, g_cpu, eps = d["x"], d["gamma"], d["eps"]
+        M, n = x_cpu.shape
+        gd = g_cpu.to(dev)
+
+        def make_set():
+            s = dict(x=x_cpu.to(dev), y=torch.empty((M, n), device=dev, dtype=torch.bfloat16),
+                     r=torch.empty((M,), device=dev, dtype=torch.float32))
+            s["args"] = (_p(s["x"]), _p(gd), _p(s["y"]), _p(s["r"]), M, n, float(eps), 0, stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_rmsnorm_fwd(*s["args"]))
+
+        def cpu_fn():
+            from oracle import fq_oracle as O
+            return O.rms_norm_forward(x_cpu, g_cpu, eps)
+
+        return Case("a2_rmsnorm_fwd", "triton_rms_norm_forward", [M, n], (2 * M * n + 2 * n, 2 * M * n + 4 * M),
+                    make_set, launch, cpu_fn)
+
+    add("a2_rmsnorm_fwd", build=rms_fwd_case)
 
     # ---------------------------------------------------------------- cfg2
     def swiglu_fwd_case(name="cfg2", pow2=False):
@@ -565,7 +593,7 @@ def load_traffic_table():
 
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
-       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "a8_blockwise", "a8_group", "a8_batch_blockwise",
+       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg1_mode0", "cfg5_mode0", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router",
        "stream_read", "stream_copy"]
 

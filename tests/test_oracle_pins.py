@@ -387,3 +387,46 @@ def test_compare_rules():
     assert rep.max_step == 2 and rep.identical == 2  # +0/-0 identical on the value line
     with pytest.raises(AssertionError):
         C.assert_codes(codes, other)
+
+
+# ---------------------------------------------------------------------------
+# the fp64 "truth" used by the GPU scale tests: the torch oracle must lie inside
+# the fp32 error bound it derives, and a scale a few ulp further out must not
+# ---------------------------------------------------------------------------
+def test_truth_bounds_hold_for_the_oracle_and_reject_a_wrong_scale():
+    from tests import truth as T
+
+    g = torch.Generator().manual_seed(77)
+    # RMSNorm + quant
+    x = (torch.randn(256, 512, generator=g) ** 3).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(512, generator=g)).to(torch.bfloat16)
+    ref = O.rms_norm_and_block_quant_forward(x, w, 1e-6)
+    y, err, r64 = T.rmsnorm_values(x, w, 1e-6)
+    sr, br, sc, bc = T.scale_bounds(y, err)
+    assert bool(((ref[1].double() - sr).abs() <= br).all()) and bool(((ref[4].double() - sc).abs() <= bc).all())
+    assert bool(((ref[2].double() - r64).abs() <= 5.5 * T.U * r64).all())
+    # a scale 20 ulp away is outside the bound (the bound is not vacuous)
+    off = (ref[1].view(torch.int32) + 20).view(torch.float32)
+    assert not bool(((off.double() - sr).abs() <= br).all())
+    # SwiGLU forward and backward, per-expert packing included
+    x2 = torch.randn(300, 512, generator=g).to(torch.bfloat16)
+    dy = (1e-2 * torch.randn(300, 256, generator=g)).to(torch.bfloat16)
+    wt = torch.rand(300, 1, generator=g)
+    counts = [130, 0, 7, 163]
+    rf = O.batch_weighted_silu_and_block_quant_forward(x2, wt, counts, False)
+    yv, ye = T.swiglu_values(x2, wt)
+    sr, br, sc, bc = T.scale_bounds_per_expert(yv, ye, counts)
+    assert bool(((rf[1].double() - sr).abs() <= br).all()) and bool(((rf[3].double() - sc).abs() <= bc).all())
+    rb = O.batch_weighted_silu_and_block_quant_backward(dy, x2, wt, counts, False)
+    dv, de, dw64 = T.swiglu_grad_values(dy, x2, wt)
+    sr, br, sc, bc = T.scale_bounds_per_expert(dv, de, counts)
+    assert bool(((rb[1].double() - sr).abs() <= br).all()) and bool(((rb[4].double() - sc).abs() <= bc).all())
+    torch.testing.assert_close(rb[2].view(-1).double(), dw64, rtol=1e-5, atol=1e-7)
+    # the fp64 derivative itself, against autograd in fp64
+    xd = x2.double().requires_grad_()
+    (torch.sigmoid(xd[:, :256]) * xd[:, :256] * xd[:, 256:] * wt.double()).backward(dy.double())
+    torch.testing.assert_close(dv, xd.grad, rtol=1e-12, atol=1e-14)
+    # a cancelling element gets a wider bound than its neighbours: x1 = -1.2785 makes 1 + x1 (1 - s) ~ 0
+    xc = torch.tensor([[-1.2785, 0.5, 1.0, 1.0]], dtype=torch.float64)
+    dvc, dec, _ = T.swiglu_grad_values(torch.ones(1, 2, dtype=torch.float64), xc)
+    assert float(dec[0, 0] / dvc[0, 0].abs()) > 50 * float(dec[0, 1] / dvc[0, 1].abs())
