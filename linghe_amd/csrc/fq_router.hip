@@ -35,7 +35,7 @@
 // (lanes 32-63), so that a lane's eight B loads of a block cover one contiguous
 // 128-byte line of its W row; the 32x32 result has column l%32 and rows
 // (v/4)*8 + (l/32)*4 + v%4 in register v.
-#include "fq_device.cuh"
+#include "fq_device.hpp"
 #include "fq_launch.h"
 
 namespace fq {

@@ -13,7 +13,7 @@
 // processed.
 #include <mutex>
 
-#include "fq_device.cuh"
+#include "fq_device.hpp"
 #include "fq_launch.h"
 
 namespace fq {

@@ -4,7 +4,7 @@
 // configuration (the measured ceiling the kernels are compared with, beside the
 // 8 TB/s of the data sheet); on a known size it calibrates the profiler's
 // FETCH_SIZE / WRITE_SIZE counters.
-#include "fq_device.cuh"
+#include "fq_device.hpp"
 #include "fq_launch.h"
 
 namespace fq {

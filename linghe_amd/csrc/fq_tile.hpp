@@ -12,7 +12,7 @@
 // and a thread owns RPT consecutive rows of 8 columns (the transposed codes of
 // one column are RPT consecutive bytes -> one LDS store).
 #pragma once
-#include "fq_device.cuh"
+#include "fq_device.hpp"
 
 namespace fq {
 
@@ -85,7 +85,7 @@ __device__ __forceinline__ void wave_column_max(const float (&cm)[8], float& lo,
 typedef uint32_t u32x2_any __attribute__((ext_vector_type(2), aligned(1)));
 typedef uint32_t u32_any __attribute__((aligned(1)));
 typedef uint16_t u16_any __attribute__((aligned(1)));
-// STREAM: with the non-temporal hint (fq_device.cuh)
+// STREAM: with the non-temporal hint (fq_device.hpp)
 typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(1)));
 template <bool STREAM>
 __device__ __forceinline__ void store16_any(uint8_t* dst, const uint4& v) {

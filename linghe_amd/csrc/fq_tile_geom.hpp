@@ -1,7 +1,7 @@
 // Where a 128x128 tile of a launch lives: its rows, its column block and the
 // offsets of its four outputs, for the single-matrix and the per-expert forms.
 #pragma once
-#include "fq_tile.cuh"
+#include "fq_tile.hpp"
 
 namespace fq {
 

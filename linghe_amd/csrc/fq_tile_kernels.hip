@@ -4,7 +4,7 @@
 //   silu_quant_bwd       SwiGLU backward + quant      (linghe/utils/silu.py:338-464, 1097-1393)
 //   rmsnorm_quant_tile   (x*rstd)*gamma + quant with a given rstd
 //                                                    (linghe/utils/norm.py:301-340)
-#include "fq_tile_geom.cuh"
+#include "fq_tile_geom.hpp"
 #include "fq_launch.h"
 
 // Cache policy per kernel, chosen by measurement (cold inputs, MI355X).
