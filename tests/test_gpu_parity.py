@@ -149,6 +149,25 @@ def test_batch_blockwise_quant(gpu, counts):
         check_quant_pair("batch_blockwise.col", ref[2], ref[3], qt, st, **EXACT)
 
 
+def test_batch_blockwise_quant_more_than_1024_experts(gpu):
+    """The per-expert tile lookup fetches the counts of 1024 experts at a time: with more
+    experts than that (most of them tiny or empty) it takes a second round."""
+    from linghe_amd.quant.block import triton_batch_blockwise_quant
+
+    announce("batch_blockwise_quant, 1300 experts")
+    rng = torch.Generator().manual_seed(15)
+    counts = [int(c) for c in torch.randint(0, 40, (1300,), generator=rng)]
+    counts[5], counts[1029], counts[1299] = 300, 257, 129
+    M, N = sum(counts), 256
+    x = randn_bf16(gen(16), M, N)
+    ref = O.batch_blockwise_quant(x, counts, False)
+    cnt = torch.tensor(counts, dtype=torch.int32, device=gpu)
+    q, s, qt, st = triton_batch_blockwise_quant(_dev(x, gpu), cnt, counts)
+    torch.cuda.synchronize()
+    check_quant_pair("batch_blockwise.1300.row", ref[0], ref[1], q, s, **EXACT)
+    check_quant_pair("batch_blockwise.1300.col", ref[2], ref[3], qt, st, **EXACT)
+
+
 # ------------------------------------------------------------------ RMSNorm
 @pytest.mark.parametrize("M,N", [(1024, 2048), (1024, 1664), (208, 1664), (512, 4096), (256, 8192),
                                  (300, 512), (64, 7168), (130, 1536), (96, 1024), (40, 128), (3, 2048),
