@@ -127,6 +127,8 @@ def build_cases(names, dev):
     # output_mode 0 (row-wise codes only: the first forward of a layer that will be recomputed)
     add("cfg1_mode0", build=lambda: rms_quant_case("cfg1_mode0", configs.cfg1_rmsnorm_quant(), 0))
     add("cfg5_mode0", build=lambda: rms_quant_case("cfg5_mode0", cfg5(), 0))
+    # output_mode 1 at cfg1's size (cfg5c is the same at cfg5's): the recomputed forward
+    add("cfg1_mode1", build=lambda: rms_quant_case("cfg1_mode1", configs.cfg1_rmsnorm_quant(), 1))
 
     # ---------------------------------------------------------------- bf16 RMSNorm forward (a2)
     def rms_fwd_case():
@@ -593,7 +595,7 @@ def load_traffic_table():
 
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
-       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg1_mode0", "cfg5_mode0", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
+       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router",
        "stream_read", "stream_copy"]
 

@@ -12,17 +12,25 @@
 //   codes, bit 1: row-wise codes).  With it the outputs do not displace inputs from L2
 //   and the memory-side cache: gather+pad+quant 75 -> 55 us, RMSNorm+quant after the
 //   statistic pass 25 -> 21 us (8192 x 2048) and 146 -> 122 us (16384 x 7168).  The
-//   SwiGLU backward is 3-7 % slower when its transposed stores carry it, the plain
-//   blockwise quantisers 10-17 % slower with any of it.  Transposed rows that do not start
+//   SwiGLU backward is 3-7 % slower when its transposed stores carry it; the plain
+//   blockwise quantiser takes none (13.2 us at 8192 x 2048 against 14.2-16.1 with any), its
+//   per-expert form (suffix _B) the transposed stores only (31.5 us against 39.2 without, 32.7
+//   with the row-wise codes only and 36.3 with both); the RMSNorm tile kernel with the
+//   statistic given (transposed output only, x read once: nothing to protect) none
+//   (16384 x 7168: 66.6 -> 59.5 us).  Transposed rows that do not start
 //   on 16-byte boundaries (M or a per-expert count that is not a multiple of 16) are where
 //   the hint on the transposed stores costs most: the SwiGLU forward takes 100 instead of
 //   70 us at 16300 x 3584 with it (and gains 3 % at 8192 x 2048), so it keeps the hint on
 //   the row-wise codes only; the RMSNorm tile kernel gains 18 % from it on aligned rows
 //   and loses 8 % on unaligned ones.
 //   FQ_LDNT_<kernel>: the bulk loads carry it (3-5 % on the SwiGLU kernels and the
-//   RMSNorm tile kernel, nothing on the plain quantisers).
+//   RMSNorm tile kernel, 12 % on the plain blockwise quantiser, 6 % on its per-expert form;
+//   the gathered rows, which several experts read, are 27 % slower with it).
 #ifndef FQ_NT_BLOCKWISE
 #define FQ_NT_BLOCKWISE 0
+#endif
+#ifndef FQ_NT_BLOCKWISE_B
+#define FQ_NT_BLOCKWISE_B 1
 #endif
 #ifndef FQ_NT_PERMUTE
 #define FQ_NT_PERMUTE 3
@@ -33,8 +41,18 @@
 #ifndef FQ_NT_SILU_BWD
 #define FQ_NT_SILU_BWD 2
 #endif
+#ifndef FQ_NT_SILU_FWD_B
+#define FQ_NT_SILU_FWD_B 2
+#endif
+#ifndef FQ_NT_SILU_BWD_B
+#define FQ_NT_SILU_BWD_B 2
+#endif
 #ifndef FQ_NT_RMSNORM
 #define FQ_NT_RMSNORM 3
+#endif
+// transposed output only (the statistic is given, x is read once: nothing to protect)
+#ifndef FQ_NT_RMSNORM_T
+#define FQ_NT_RMSNORM_T 0
 #endif
 //   FQ_LEAN_BLOCKWISE: the lean form of the quantiser and of the tile loads (scalar
 //   bases, paired column-maximum reduction; every other tile kernel uses it, -3 to -9 %)
@@ -44,7 +62,10 @@
 #define FQ_LEAN_BLOCKWISE 0
 #endif
 #ifndef FQ_LDNT_BLOCKWISE
-#define FQ_LDNT_BLOCKWISE 0
+#define FQ_LDNT_BLOCKWISE 1
+#endif
+#ifndef FQ_LDNT_BLOCKWISE_B
+#define FQ_LDNT_BLOCKWISE_B 1
 #endif
 #ifndef FQ_LDNT_PERMUTE
 #define FQ_LDNT_PERMUTE 0
@@ -54,6 +75,12 @@
 #endif
 #ifndef FQ_LDNT_SILU_BWD
 #define FQ_LDNT_SILU_BWD 1
+#endif
+#ifndef FQ_LDNT_SILU_FWD_B
+#define FQ_LDNT_SILU_FWD_B 1
+#endif
+#ifndef FQ_LDNT_SILU_BWD_B
+#define FQ_LDNT_SILU_BWD_B 1
 #endif
 #ifndef FQ_LDNT_RMSNORM
 #define FQ_LDNT_RMSNORM 1
@@ -82,11 +109,14 @@ __global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __
   const TileGeom g = resolve_tile<BATCHED>(M, N / kGroup, N, batch);
   if (!g.valid) return;
   uint4 raw[RPT];
-  load_rows<RPT, FQ_LDNT_BLOCKWISE != 0, BATCHED || FQ_LEAN_BLOCKWISE != 0>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
+  constexpr bool LDNT = (BATCHED ? FQ_LDNT_BLOCKWISE_B : FQ_LDNT_BLOCKWISE) != 0;
+  constexpr int NT = BATCHED ? FQ_NT_BLOCKWISE_B : FQ_NT_BLOCKWISE;
+  constexpr bool LEAN = BATCHED || FQ_LEAN_BLOCKWISE != 0;
+  load_rows<RPT, LDNT, LEAN>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
-  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_BLOCKWISE, BATCHED || FQ_LEAN_BLOCKWISE != 0>(v, make_out(out, g, N, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, NT, LEAN>(v, make_out(out, g, N, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -163,8 +193,10 @@ __global__ __launch_bounds__(2048 / FQ_RPT_FWD) void silu_quant_fwd_kernel(const
   const int64_t ld = 2 * (int64_t)n;
   uint4 r1[RPT], r2[RPT];
   const uint16_t* p = x + g.row0 * ld + (int64_t)g.cb * kGroup;
-  load_rows<RPT, FQ_LDNT_SILU_FWD != 0>(p, ld, g.rows_valid, r1);
-  load_rows<RPT, FQ_LDNT_SILU_FWD != 0>(p + n, ld, g.rows_valid, r2);
+  constexpr bool LDNT = (BATCHED ? FQ_LDNT_SILU_FWD_B : FQ_LDNT_SILU_FWD) != 0;
+  constexpr int NT = BATCHED ? FQ_NT_SILU_FWD_B : FQ_NT_SILU_FWD;
+  load_rows<RPT, LDNT>(p, ld, g.rows_valid, r1);
+  load_rows<RPT, LDNT>(p + n, ld, g.rows_valid, r2);
   const int rg = threadIdx.x >> 4;
   float v[RPT][8];
 #pragma unroll
@@ -190,7 +222,7 @@ __global__ __launch_bounds__(2048 / FQ_RPT_FWD) void silu_quant_fwd_kernel(const
       }
     }
   }
-  quantize_tile<KIND, ROUND, MODE, RPT, FQ_NT_SILU_FWD>(v, make_out(out, g, n, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, NT>(v, make_out(out, g, n, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -211,9 +243,11 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   if (!g.valid) return;
   uint4 r1[RPT], r2[RPT], rgd[RPT];
   const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
-  load_rows<RPT, FQ_LDNT_SILU_BWD != 0>(p, N, g.rows_valid, r1);
-  load_rows<RPT, FQ_LDNT_SILU_BWD != 0>(p + n, N, g.rows_valid, r2);
-  load_rows<RPT, FQ_LDNT_SILU_BWD != 0>(gr + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, rgd);
+  constexpr bool LDNT = (BATCHED ? FQ_LDNT_SILU_BWD_B : FQ_LDNT_SILU_BWD) != 0;
+  constexpr int NT = BATCHED ? FQ_NT_SILU_BWD_B : FQ_NT_SILU_BWD;
+  load_rows<RPT, LDNT>(p, N, g.rows_valid, r1);
+  load_rows<RPT, LDNT>(p + n, N, g.rows_valid, r2);
+  load_rows<RPT, LDNT>(gr + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, rgd);
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
   float d[2][RPT][8];  // dx1, dx2
@@ -265,15 +299,15 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
     // with it, so it quantises one tile after the other.
     __shared__ TileShared<RPT, 2> sh;
     const TileOut outs[2] = {make_out(out, g, N, g.cb), make_out(out, g, N, nb + g.cb)};
-    quantize_tiles<KIND, ROUND, 2, RPT, FQ_NT_SILU_BWD, true, 2>(d, outs, sh);
+    quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 2>(d, outs, sh);
   } else {
     __shared__ TileShared<RPT> sh;
     const TileOut o1[1] = {make_out(out, g, N, g.cb)};
     const TileOut o2[1] = {make_out(out, g, N, nb + g.cb)};
     const float (&dx1)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(d[0]);
     const float (&dx2)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(d[1]);
-    quantize_tiles<KIND, ROUND, 2, RPT, FQ_NT_SILU_BWD, true, 1, true>(dx1, o1, sh);
-    quantize_tiles<KIND, ROUND, 2, RPT, FQ_NT_SILU_BWD, true, 1, false>(dx2, o2, sh);
+    quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 1, true>(dx1, o1, sh);
+    quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 1, false>(dx2, o2, sh);
   }
 }
 
@@ -422,7 +456,7 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
         FQ_DISPATCH_BOOL(aligned_rows, A,
-          hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD, A ? FQ_NT_RMSNORM : (FQ_NT_RMSNORM & 2)>), grid,
+          hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD, MD == 1 ? FQ_NT_RMSNORM_T : A ? FQ_NT_RMSNORM : (FQ_NT_RMSNORM & 2)>), grid,
                              block, 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, rstd, out, M, n,
                              remap);))))
   return hipGetLastError();
