@@ -156,17 +156,20 @@ def build_cases(names, dev):
     add("a2_rmsnorm_fwd", build=rms_fwd_case)
 
     # ---------------------------------------------------------------- cfg2
-    def swiglu_fwd_case(name="cfg2", pow2=False):
+    def swiglu_fwd_case(name="cfg2", pow2=False, mode=2):
         x_cpu = configs.cfg2_swiglu_fwd()["x"]
         M, N = x_cpu.shape
         n = N // 2
 
         def make_set():
-            s = dict(x=x_cpu.to(dev), q=torch.empty((M, n), device=dev, dtype=FP8),
-                     s=torch.empty((n // 128, M), device=dev, dtype=torch.float32),
-                     qt=torch.empty((n, M), device=dev, dtype=FP8),
-                     st=torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32))
-            s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, int(pow2), 2,
+            s = dict(x=x_cpu.to(dev), q=None, s=None, qt=None, st=None)
+            if mode != 1:
+                s["q"] = torch.empty((M, n), device=dev, dtype=FP8)
+                s["s"] = torch.empty((n // 128, M), device=dev, dtype=torch.float32)
+            if mode != 0:
+                s["qt"] = torch.empty((n, M), device=dev, dtype=FP8)
+                s["st"] = torch.empty(((M + 127) // 128, n), device=dev, dtype=torch.float32)
+            s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, int(pow2), mode,
                          _lib.FQ_E4M3, stream)
             return s
 
@@ -177,12 +180,15 @@ def build_cases(names, dev):
             from oracle import fq_oracle as O
             return O.silu_and_block_quant_forward(x_cpu, pow2)
 
-        return Case(name, "triton_silu_and_block_quant_forward(output_mode=2%s)" % (", round_scale=True" if pow2 else ""),
+        return Case(name, "triton_silu_and_block_quant_forward(output_mode=%d%s)" % (mode, ", round_scale=True" if pow2 else ""),
                     [M, N],
-                    configs.rw_swiglu_fwd(M, n), make_set, launch, cpu_fn)
+                    configs.rw_swiglu_fwd(M, n, mode), make_set, launch, cpu_fn)
 
     add("cfg2", build=swiglu_fwd_case)
     add("cfg2_pow2", build=lambda: swiglu_fwd_case("cfg2_pow2", True))
+    # one layout only: what a recomputed layer asks for (row-wise in the forward, transposed in the recomputation)
+    add("cfg2_mode0", build=lambda: swiglu_fwd_case("cfg2_mode0", False, 0))
+    add("cfg2_mode1", build=lambda: swiglu_fwd_case("cfg2_mode1", False, 1))
 
     # ---------------------------------------------------------------- cfg3 (+ backward)
     def batched_case(backward):
@@ -595,7 +601,7 @@ def load_traffic_table():
 
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
-       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
+       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router",
        "stream_read", "stream_copy"]
 

@@ -120,8 +120,10 @@ def rw_rmsnorm_quant(M, n, mode=2):
     return x, row + col + 4 * M
 
 
-def rw_swiglu_fwd(M, n):
-    return 2 * M * 2 * n, 2 * M * n + 4 * (n // 128) * M + 4 * ((M + 127) // 128) * n
+def rw_swiglu_fwd(M, n, mode=2):
+    row = M * n + 4 * (n // 128) * M
+    col = M * n + 4 * ((M + 127) // 128) * n
+    return 2 * M * 2 * n, (row if mode != 1 else 0) + (col if mode != 0 else 0)
 
 
 def rw_swiglu_bwd(M, n):

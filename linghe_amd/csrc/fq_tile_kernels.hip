@@ -41,6 +41,12 @@
 #ifndef FQ_NT_SILU_BWD
 #define FQ_NT_SILU_BWD 2
 #endif
+#ifndef FQ_NT_SILU_FWD_M0
+#define FQ_NT_SILU_FWD_M0 2
+#endif
+#ifndef FQ_NT_SILU_FWD_M1
+#define FQ_NT_SILU_FWD_M1 1
+#endif
 #ifndef FQ_NT_SILU_FWD_B
 #define FQ_NT_SILU_FWD_B 2
 #endif
@@ -194,7 +200,7 @@ __global__ __launch_bounds__(2048 / FQ_RPT_FWD) void silu_quant_fwd_kernel(const
   uint4 r1[RPT], r2[RPT];
   const uint16_t* p = x + g.row0 * ld + (int64_t)g.cb * kGroup;
   constexpr bool LDNT = (BATCHED ? FQ_LDNT_SILU_FWD_B : FQ_LDNT_SILU_FWD) != 0;
-  constexpr int NT = BATCHED ? FQ_NT_SILU_FWD_B : FQ_NT_SILU_FWD;
+  constexpr int NT = MODE == 0 ? FQ_NT_SILU_FWD_M0 : MODE == 1 ? FQ_NT_SILU_FWD_M1 : BATCHED ? FQ_NT_SILU_FWD_B : FQ_NT_SILU_FWD;
   load_rows<RPT, LDNT>(p, ld, g.rows_valid, r1);
   load_rows<RPT, LDNT>(p + n, ld, g.rows_valid, r2);
   const int rg = threadIdx.x >> 4;
