@@ -315,6 +315,23 @@ __device__ __forceinline__ double wave_sum_d(double v) {
   return v;
 }
 
+// Scheduling fences for the register allocator.  The compiler likes to widen the packed bf16
+// rows of a tile as soon as they arrive, long before the arithmetic that uses them; the fp32
+// copies (twice the registers) then sit beside the results of earlier rows and push a kernel
+// over its register cap.  fence_values / fence_packed cost no instruction: they are empty
+// volatile asm statements (which keep their order among themselves) that claim to rewrite
+// their operands, so whatever is computed from a fenced packed row starts after the fenced
+// results before it are complete.
+__device__ __forceinline__ void fence_values(float (&v)[8]) {
+  asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+}
+__device__ __forceinline__ void fence_packed(uint4& p) {
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));  // one 128-bit operand: the four dwords stay a tuple
+  u32x4 t = __builtin_bit_cast(u32x4, p);
+  asm volatile("" : "+v"(t));
+  p = __builtin_bit_cast(uint4, t);
+}
+
 // sigmoid(x) = 1 / (1 + exp(-x)):
 //   exp(-x) = exp2(-x*log2(e)) with v_exp_f32 (1 ulp). A single fp32 product
 //   x * -log2(e) would round the exponent and cost up to |x|*4e-8 of relative error

@@ -96,6 +96,9 @@
 // thread spread the per-thread overhead over twice the elements: the RMSNorm tile
 // kernel (93 registers, five 256-thread workgroups per CU) gains 3-4 %; the SwiGLU
 // forward needs 135 registers in that shape and loses 5 %.
+#ifndef FQ_BWD_PIN
+#define FQ_BWD_PIN 1
+#endif
 #ifndef FQ_RPT_FWD
 #define FQ_RPT_FWD 4
 #endif
@@ -265,6 +268,20 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   if ((threadIdx.x >> 6) * (4 * RPT) < g.rows_valid) {  // waves beyond the last row of a partial tile keep zeros
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
+#if FQ_BWD_PIN
+      if constexpr (BATCHED || FQ_BWD_PIN > 1) {
+        // row s is widened after row s-1 is done (see fence_values): 136 -> 122 registers in the
+        // per-expert form, which was capped at 128 and spilled 8 (16 KB of scratch traffic per tile,
+        // a quarter of the output again in HBM writes: 97.1 -> 89.1 us at 65536 x 1024, 256 experts)
+        if (s > 0) {
+          fence_values(d[0][s - 1]);
+          fence_values(d[1][s - 1]);
+          fence_packed(r1[s]);
+          fence_packed(r2[s]);
+          fence_packed(rgd[s]);
+        }
+      }
+#endif
       float a[8], b[8], go[8];
       unpack8(r1[s], a);
       unpack8(r2[s], b);
