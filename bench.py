@@ -6,8 +6,10 @@
 A "step" is one call of the entry point of a configuration on one batch of
 synthetic (seeded) input that is already resident in HBM.  Calls go through
 the C ABI with preallocated outputs; K steps are timed between two events on
-the launch stream, R times over, and the median loop is reported (with the
-fastest and slowest).  Buffers rotate over enough copies to exceed twice the
+the launch stream (HIP events without the system-scope fence), R times over,
+and the median loop is reported (with the fastest and slowest); every timed
+loop follows, in the stream, untimed calls of the same entry point that keep
+the device busy for --settle-us (1.5 ms) first.  Buffers rotate over enough copies to exceed twice the
 256 MB Infinity Cache, so the figure is an HBM figure ("cold"); the same loop
 on one fixed set of buffers gives the cache-resident ("hot") figure.
 
@@ -505,23 +507,88 @@ def build_cases(names, dev):
     return cases
 
 
-def time_loop(launch, sets, steps, warmup, repeats):
+class TimingEvents:
+    """A pair of HIP events created with hipEventDisableSystemFence and recorded on the launch
+    stream.  A default event performs a system-scope fence (cache write-back and invalidation)
+    when it is recorded; HIP documents this flag for events that only measure time.  With default
+    events every timed loop carries 25-85 us of fence work that is not the kernels' (a 20-call loop
+    of the SwiGLU backward reads 37.2 us per call where the kernel trace of the same loop shows
+    20 dispatches of 33.3-34.9 us back to back)."""
+    _hip = None
+
+    def __init__(self, stream):
+        import ctypes
+        if TimingEvents._hip is None:
+            TimingEvents._hip = ctypes.CDLL("libamdhip64.so")
+        self.c, self.hip, self.stream = ctypes, TimingEvents._hip, ctypes.c_void_p(stream)
+        self.a, self.b = ctypes.c_void_p(), ctypes.c_void_p()
+        for e in (self.a, self.b):
+            self._ok(self.hip.hipEventCreateWithFlags(ctypes.byref(e), ctypes.c_uint(0x20000000)))
+
+    def _ok(self, rc):
+        if rc != 0:
+            raise RuntimeError("HIP event call failed with error %d" % rc)
+
+    def start(self):
+        self._ok(self.hip.hipEventRecord(self.a, self.stream))
+
+    def stop(self):
+        self._ok(self.hip.hipEventRecord(self.b, self.stream))
+
+    def elapsed_us(self):
+        ms = self.c.c_float()
+        self._ok(self.hip.hipEventSynchronize(self.b))
+        self._ok(self.hip.hipEventElapsedTime(self.c.byref(ms), self.a, self.b))
+        return ms.value * 1000.0
+
+    def close(self):
+        for e in (self.a, self.b):
+            self.hip.hipEventDestroy(e)
+
+
+SETTLE_US = 1500.0  # see time_loop; --settle-us 0 turns it off
+
+
+def time_loop(launch, sets, steps, warmup, repeats, settle_us=None):
     """us per call, one figure per repeat: `steps` back-to-back launches between two
-    events on the launch stream (the current torch stream), rotating over `sets`."""
+    events on the launch stream (the current torch stream), rotating over `sets`.
+
+    Every repeat is: synchronize, pre-roll, start event, exactly `steps` calls, stop event,
+    synchronize.  The pre-roll is untimed calls of the same entry point, enqueued right in
+    front of the start event, enough of them to keep the device busy for `settle_us`: a loop
+    that starts on a device that has been mostly idle runs at a lower rate for its first
+    millisecond or so (20 calls of the SwiGLU backward read 36-39 us per call that way, 33.7-34.0
+    behind a pre-roll of 30 calls or more, and 33.9 in loops of 100-300 calls with no pre-roll at
+    all; the kernel trace of a slow loop shows the same 33-35 us dispatches, so the difference is
+    not inside the kernels), so what a short loop measures from idle is the device waking up, not
+    the steady state the path runs in."""
     k = len(sets)
     for i in range(warmup):
         launch(sets[i % k])
+    ev = TimingEvents(torch.cuda.current_stream().cuda_stream)
+    settle_us = SETTLE_US if settle_us is None else settle_us
+    preroll = 0
+    if settle_us > 0:
+        torch.cuda.synchronize()
+        ev.start()
+        for i in range(8):
+            launch(sets[i % k])
+        ev.stop()
+        torch.cuda.synchronize()
+        preroll = max(warmup, min(2000, int(settle_us / max(ev.elapsed_us() / 8, 0.5)) + 1))
     out = []
     for _ in range(repeats):
         torch.cuda.synchronize()
-        start = torch.cuda.Event(enable_timing=True)
-        end = torch.cuda.Event(enable_timing=True)
-        start.record()
-        for i in range(steps):
+        for i in range(preroll):
             launch(sets[i % k])
-        end.record()
+        ev.start()
+        for i in range(steps):
+            launch(sets[(preroll + i) % k])
+        ev.stop()
         torch.cuda.synchronize()
-        out.append(start.elapsed_time(end) * 1000.0 / steps)
+        out.append(ev.elapsed_us() / steps)
+    ev.close()
+    time_loop.last_preroll = preroll
     return sorted(out)
 
 
@@ -607,11 +674,14 @@ ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "
 
 
 def main():
+    global SETTLE_US
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--repeats", type=int, default=7, help="timed loops of --steps calls per figure; the median is reported")
+    ap.add_argument("--settle-us", type=float, default=SETTLE_US,
+                    help="untimed pre-roll in front of every timed loop, in us of device time (0: loops start on an idle device)")
     ap.add_argument("--configs", default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the no-work stream kernel on each config's bytes")
@@ -619,6 +689,7 @@ def main():
                     help="profiling aid: run only the named configs and print their results without the headline line")
     ap.add_argument("--hot-only", action="store_true", help="profiling aid: one buffer set, no rotation")
     args = ap.parse_args()
+    SETTLE_US = max(0.0, args.settle_us)
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (every row block / expert is independent, "
               "there is no collective to time); --gpus must be 1", file=sys.stderr)
@@ -647,6 +718,7 @@ def main():
                                                    min(3, args.repeats))
         med, trimmed = time_single_calls(case, case.sets, max(10, min(args.steps, 200)), min(args.warmup, 10))
         cold = time_loop(case.launch, case.sets, args.steps, args.warmup, args.repeats)
+        preroll = time_loop.last_preroll
         if hot is None:
             hot = cold
         us = median(cold)
@@ -654,7 +726,8 @@ def main():
         r = dict(entry=case.entry, shape=case.shape, algorithmic_bytes=case.algo_bytes,
                  algorithmic_bytes_read=case.read_bytes, algorithmic_bytes_written=case.write_bytes,
                  us_per_call=round(us, 3), us_per_call_min=round(cold[0], 3), us_per_call_max=round(cold[-1], 3),
-                 timed_loops=len(cold), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
+                 timed_loops=len(cold), preroll_calls=preroll,
+                 gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
                  us_per_call_hot=round(median(hot), 3), gb_per_s_hot=round(case.algo_bytes / median(hot) / 1e3, 1),
                  us_single_call_median=round(med, 3), us_single_call_trimmed_mean=round(trimmed, 3),
                  buffer_sets=len(case.sets))
@@ -710,7 +783,9 @@ def main():
         "config": {"workload": "cfg1: RMSNorm + 1x128/128x1 e4m3 blockwise quant forward, x bf16 [8192,2048], "
                                "output_mode 2, round_scale False, buffers rotated beyond the Infinity Cache; "
                                "bf16 in, fp32 arithmetic, fp8 + fp32 scales out; value = median of %d loops of "
-                               "%d calls" % (head["timed_loops"], args.steps),
+                               "%d calls, each loop behind %d untimed calls of the same entry point that keep the device "
+                               "busy for %.1f ms before the start event (--settle-us 0: loops start on an idle device)"
+                               % (head["timed_loops"], args.steps, head["preroll_calls"], SETTLE_US / 1000.0),
                    "entry": head["entry"]},
         "roofline": roofline,
         "configs": results,
