@@ -549,7 +549,7 @@ class TimingEvents:
 SETTLE_US = 1500.0  # see time_loop; --settle-us 0 turns it off
 
 
-def time_loop(launch, sets, steps, warmup, repeats, settle_us=None):
+def time_loop(launch, sets, steps, warmup, repeats, settle_us=None, idle_gap_s=0.0):
     """us per call, one figure per repeat: `steps` back-to-back launches between two
     events on the launch stream (the current torch stream), rotating over `sets`.
 
@@ -579,6 +579,8 @@ def time_loop(launch, sets, steps, warmup, repeats, settle_us=None):
     out = []
     for _ in range(repeats):
         torch.cuda.synchronize()
+        if idle_gap_s > 0:
+            time.sleep(idle_gap_s)  # let the device go idle: the from-idle figure
         for i in range(preroll):
             launch(sets[i % k])
         ev.start()
@@ -714,6 +716,12 @@ def main():
         # the cache-resident loops and the single-call samples run first: by the time the
         # headline (cold) loops start the device has been busy for a few milliseconds and
         # its clocks have settled (the first loop after host-side set-up reads up to 10 % slow)
+        # for the record, the headline configuration is also timed the plain way first: warm-up, then
+        # loops of `steps` calls that each start on a device left idle for 20 ms
+        idle = None
+        if name == "cfg1" and not args.hot_only and SETTLE_US > 0:
+            idle = time_loop(case.launch, case.sets, args.steps, args.warmup, min(5, args.repeats), settle_us=0,
+                             idle_gap_s=0.02)
         hot = None if args.hot_only else time_loop(case.launch, case.sets[:1], args.steps, args.warmup,
                                                    min(3, args.repeats))
         med, trimmed = time_single_calls(case, case.sets, max(10, min(args.steps, 200)), min(args.warmup, 10))
@@ -731,6 +739,8 @@ def main():
                  us_per_call_hot=round(median(hot), 3), gb_per_s_hot=round(case.algo_bytes / median(hot) / 1e3, 1),
                  us_single_call_median=round(med, 3), us_single_call_trimmed_mean=round(trimmed, 3),
                  buffer_sets=len(case.sets))
+        if idle is not None:
+            r["us_per_call_from_idle"] = round(median(idle), 3)
         if hasattr(case, "extra"):
             r.update(case.extra)
         # the buffers of the case are released before the ceiling and the CPU leg allocate theirs
@@ -784,8 +794,10 @@ def main():
                                "output_mode 2, round_scale False, buffers rotated beyond the Infinity Cache; "
                                "bf16 in, fp32 arithmetic, fp8 + fp32 scales out; value = median of %d loops of "
                                "%d calls, each loop behind %d untimed calls of the same entry point that keep the device "
-                               "busy for %.1f ms before the start event (--settle-us 0: loops start on an idle device)"
-                               % (head["timed_loops"], args.steps, head["preroll_calls"], SETTLE_US / 1000.0),
+                               "busy for %.1f ms before the start event%s"
+                               % (head["timed_loops"], args.steps, head["preroll_calls"], SETTLE_US / 1000.0,
+                                  "; the same loops started on a device left idle for 20 ms: %.2f us/call"
+                                  % head["us_per_call_from_idle"] if "us_per_call_from_idle" in head else ""),
                    "entry": head["entry"]},
         "roofline": roofline,
         "configs": results,
