@@ -91,11 +91,13 @@
 #ifndef FQ_LDNT_RMSNORM
 #define FQ_LDNT_RMSNORM 1
 #endif
-// Rows per thread (workgroup = 2048 / RPT threads).  With the outputs streamed past
-// the caches the tile kernels are bound by vector-instruction issue, and 8 rows per
-// thread spread the per-thread overhead over twice the elements: the RMSNorm tile
-// kernel (93 registers, five 256-thread workgroups per CU) gains 3-4 %; the SwiGLU
-// forward needs 135 registers in that shape and loses 5 %.
+// Rows per thread (workgroup = 2048 / RPT threads).  8 rows per thread spread the
+// per-thread overhead over twice the elements, 4 rows per thread put twice the waves on
+// a CU.  The SwiGLU forward needs 135 registers with 8 and loses 5-9 %.  The RMSNorm tile
+// kernel measured 3-4 % ahead with 8 (93 registers, five 256-thread workgroups per CU)
+// when its division took three operations per element; with the current two it is level
+// at 16384 x 7168 (110.5 us either way, 58.9 / 58.5 us with the statistic given) and
+// 2 % behind at 8192 x 2048 (18.3 / 18.0 us), so it runs with 4.
 #ifndef FQ_BWD_PIN
 #define FQ_BWD_PIN 1
 #endif
@@ -103,7 +105,7 @@
 #define FQ_RPT_FWD 4
 #endif
 #ifndef FQ_RPT_RMS
-#define FQ_RPT_RMS 8
+#define FQ_RPT_RMS 4
 #endif
 namespace fq {
 
