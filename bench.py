@@ -19,9 +19,12 @@ measured ceiling of this device for those bytes), the HBM traffic per call
 measured with the profiler's counters (from profiles/hbm_traffic_per_config.md)
 and the torch CPU oracle timed on the host cores.
 
-Prints ONE JSON line: the headline metric is us/call of RMSNorm + 1x128 quant
-forward on bf16 [8192, 2048] (output_mode 2); the other configurations are
-listed under "configs".
+Prints ONE short JSON line on stdout (under 4000 characters): the headline
+metric is us/call of RMSNorm + 1x128 quant forward on bf16 [8192, 2048]
+(output_mode 2) with its roofline and CPU baseline; the other configurations
+appear as name -> [us, fraction of peak, fraction of the no-work kernel's rate].
+Every field of every configuration goes to gpurun_out/bench_full.json; stderr
+carries one summary line per configuration.
 """
 from __future__ import annotations
 
@@ -716,10 +719,10 @@ def main():
         # the cache-resident loops and the single-call samples run first: by the time the
         # headline (cold) loops start the device has been busy for a few milliseconds and
         # its clocks have settled (the first loop after host-side set-up reads up to 10 % slow)
-        # for the record, the headline configuration is also timed the plain way first: warm-up, then
-        # loops of `steps` calls that each start on a device left idle for 20 ms
+        # for the record, the eight headline configurations are also timed the plain way first: warm-up,
+        # then loops of `steps` calls that each start on a device left idle for 20 ms
         idle = None
-        if name == "cfg1" and not args.hot_only and SETTLE_US > 0:
+        if name in HEADLINE_CONFIGS and not args.hot_only and SETTLE_US > 0:
             idle = time_loop(case.launch, case.sets, args.steps, args.warmup, min(5, args.repeats), settle_us=0,
                              idle_gap_s=0.02)
         hot = None if args.hot_only else time_loop(case.launch, case.sets[:1], args.steps, args.warmup,
@@ -770,6 +773,47 @@ def main():
     if args.no_headline:
         print(json.dumps({"configs": results}))
         return
+    write_full_results(results, args)
+    line = headline_line(results, args.steps, args.warmup, SETTLE_US)
+    print(encode_line(line), flush=True)
+
+
+def encode_line(line):
+    """JSON text of the headline line, kept under MAX_LINE_CHARS: if it ever grows beyond, the
+    per-configuration extras go first (they are in the full results anyway), never the headline."""
+    text = json.dumps(line, separators=(",", ":"))
+    for drop in ("from_idle_us", "configs"):
+        if len(text) < MAX_LINE_CHARS:
+            break
+        line = {k: v for k, v in line.items() if k != drop}
+        text = json.dumps(line, separators=(",", ":"))
+    return text
+
+
+MAX_LINE_CHARS = 4000  # the last stdout line must fit the window a harness keeps of stdout
+HEADLINE_CONFIGS = ("cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg5a", "cfg5b", "cfg5c")
+
+
+def write_full_results(results, args):
+    """Every field of every configuration: to gpurun_out/bench_full.json, or, when that cannot be
+    written, as one JSON object per configuration on stderr.  The stdout line stays short."""
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, "bench_full.json"), "w") as f:
+            json.dump({"steps": args.steps, "warmup": args.warmup, "repeats": args.repeats,
+                       "settle_us": SETTLE_US, "configs": results}, f, indent=1)
+    except OSError as e:  # a read-only tree
+        print("[bench] bench_full.json not written: %s" % e, file=sys.stderr)
+        for name, r in results.items():
+            print("[bench-full] " + json.dumps({name: r}), file=sys.stderr)
+
+
+def headline_line(results, steps, warmup, settle_us):
+    """The ONE stdout line, built from the per-configuration results: cfg1 is the headline
+    (BASELINE metric), `configs` maps every measured configuration to
+    [us per call, fraction of the 8 TB/s peak, fraction of the no-work kernel's rate on the same
+    bytes (null when not measured)], `from_idle_us` the same loops started on an idle device."""
     head = results["cfg1"]
     roofline = {"bound": "hbm", "achieved": head["gb_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": head["frac_of_hbm_peak"], "traffic": head.get("hbm_traffic_bytes")}
@@ -782,33 +826,34 @@ def main():
         "value": head["us_per_call"],
         "unit": "us/call",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
+        "preroll_calls": head.get("preroll_calls", 0),
         "ms_per_step": round(head["us_per_call"] / 1000.0, 6),
+        "us_per_call_from_idle": head.get("us_per_call_from_idle"),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "cfg1: RMSNorm + 1x128/128x1 e4m3 blockwise quant forward, x bf16 [8192,2048], "
-                               "output_mode 2, round_scale False, buffers rotated beyond the Infinity Cache; "
-                               "bf16 in, fp32 arithmetic, fp8 + fp32 scales out; value = median of %d loops of "
-                               "%d calls, each loop behind %d untimed calls of the same entry point that keep the device "
-                               "busy for %.1f ms before the start event%s"
-                               % (head["timed_loops"], args.steps, head["preroll_calls"], SETTLE_US / 1000.0,
-                                  "; the same loops started on a device left idle for 20 ms: %.2f us/call"
-                                  % head["us_per_call_from_idle"] if "us_per_call_from_idle" in head else ""),
+                               "output_mode 2, buffers rotated beyond the Infinity Cache; value = median of %d "
+                               "loops of %d calls, each behind preroll_calls untimed calls (%.1f ms of device "
+                               "time); us_per_call_from_idle = same loops on a device idle for 20 ms"
+                               % (head.get("timed_loops", 0), steps, settle_us / 1000.0),
                    "entry": head["entry"]},
         "roofline": roofline,
-        "configs": results,
     }
     if "cpu_us_per_call" in head:
         line["cpu_baseline"] = {"value": head["cpu_us_per_call"], "unit": "us/call",
                                 "cores": head["cpu_threads"], "kind": "port",
-                                "sample": "cfg1 at full size, torch CPU oracle, 1 warm-up + min of 3 calls; "
-                                          "os.cpu_count()=%d; every other config has its own cpu_us_per_call"
-                                          % os.cpu_count()}
-    print(json.dumps(line))
+                                "sample": "cfg1 at full size, torch CPU oracle, 1 warm-up + min of 3 calls"}
+    line["configs"] = {name: [r["us_per_call"], r["frac_of_hbm_peak"], r.get("frac_of_stream")]
+                       for name, r in results.items()}
+    line["from_idle_us"] = {name: r["us_per_call_from_idle"] for name, r in results.items()
+                            if "us_per_call_from_idle" in r}
+    line["full_results"] = "gpurun_out/bench_full.json"
+    return line
 
 
 if __name__ == "__main__":
