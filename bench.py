@@ -635,23 +635,77 @@ def time_cpu(case):
     return min(runs) * 1e6
 
 
-def stream_ceiling(case, dev, stream, steps, warmup, repeats):
-    """us for the no-work kernel to read and write this configuration's algorithmic byte
-    counts, cold buffers: what the memory system alone takes for the same bytes.  The
-    better of plain and non-temporal accesses."""
-    from linghe_amd import _lib
-    rb, wb = (case.read_bytes + 15) // 16 * 16, (case.write_bytes + 15) // 16 * 16
+# Variants of the no-work kernel the ceiling is taken over: (chunks per lane, workgroups, order, hint on
+# loads, hint on stores); workgroups 0 = one step per workgroup.  The short list is what came out on top
+# somewhere in the full sweep (`--stream-sweep`, table in profiles/stream_ceiling_sweep.md).
+STREAM_VARIANTS = [
+    (4, 16384, 0, 0, 0), (4, 16384, 0, 1, 1),            # the plain form, without and with the hints
+    (8, 2048, 0, 1, 1), (8, 0, 0, 1, 1), (8, 0, 1, 1, 1), (8, 0, 0, 1, 0), (8, 2048, 1, 1, 0),
+    (4, 0, 0, 1, 1), (4, 512, 0, 1, 1), (16, 0, 0, 1, 1),
+]
+
+
+def _stream_sets(dev, rb, wb):
     n_sets = max(2, min(16, (2 * INFINITY_CACHE_BYTES + (64 << 20)) // max(1, rb + wb) + 1))
-    sink = torch.zeros(16, device=dev, dtype=torch.uint8)
-    sets = [(torch.zeros(max(rb, 16), device=dev, dtype=torch.uint8),
+    return [(torch.zeros(max(rb, 16), device=dev, dtype=torch.uint8),
              torch.empty(max(wb, 16), device=dev, dtype=torch.uint8)) for _ in range(n_sets)]
+
+
+def _time_stream_variant(variant, sets, sink, rb, wb, stream, steps, warmup, repeats):
+    from linghe_amd import _lib
+    cpl, wgs, order, ntl, nts = variant
+
+    def launch(s):
+        _lib.check(_lib.lib.fq_stream_rw_variant(s[0].data_ptr(), rb, s[1].data_ptr(), wb, sink.data_ptr(), cpl, wgs,
+                                                 order, ntl, nts, stream))
+    return median(time_loop(launch, sets, steps, warmup, repeats))
+
+
+def stream_ceiling(case, dev, stream, steps, warmup, repeats):
+    """(us, variant) for the no-work kernel to read and write this configuration's algorithmic byte
+    counts, cold buffers: what the memory system alone takes for the same bytes.  The fastest of
+    STREAM_VARIANTS."""
+    rb, wb = (case.read_bytes + 15) // 16 * 16, (case.write_bytes + 15) // 16 * 16
+    sink = torch.zeros(16, device=dev, dtype=torch.uint8)
+    sets = _stream_sets(dev, rb, wb)
     best = None
-    for nt in (0, 1):
-        def launch(s, nt=nt):
-            _lib.check(_lib.lib.fq_stream_rw(s[0].data_ptr(), rb, s[1].data_ptr(), wb, sink.data_ptr(), nt, stream))
-        t = median(time_loop(launch, sets, steps, warmup, repeats))
-        best = t if best is None else min(best, t)
+    for v in STREAM_VARIANTS:
+        t = _time_stream_variant(v, sets, sink, rb, wb, stream, steps, warmup, repeats)
+        if best is None or t < best[0]:
+            best = (t, v)
     return best
+
+
+def stream_sweep(dev, stream, steps, warmup, repeats):
+    """Every variant of the no-work kernel on the byte counts of cfg1, cfg2 and cfg5a (read MB, write MB),
+    cold buffers: a markdown table on stdout (the basis of STREAM_VARIANTS)."""
+    from linghe_amd import configs
+    sizes = [("cfg1", configs.rw_rmsnorm_quant(8192, 2048, 2)), ("cfg2", configs.rw_swiglu_fwd(8192, 2048, 2)),
+             ("cfg5a", configs.rw_rmsnorm_bwd(16384, 7168))]
+    variants = [(c, w, o, l, st) for c in (4, 8, 16) for w in (256, 512, 1024, 2048, 0) for o in (0, 1, 2)
+                for l in (0, 1) for st in (0, 1)]
+    variants.insert(0, (4, 16384, 0, 0, 0))
+    variants.insert(1, (4, 16384, 0, 1, 1))
+    cols = {}
+    for name, (rb, wb) in sizes:
+        rb, wb = (rb + 15) // 16 * 16, (wb + 15) // 16 * 16
+        sink = torch.zeros(16, device=dev, dtype=torch.uint8)
+        sets = _stream_sets(dev, rb, wb)
+        cols[name] = [_time_stream_variant(v, sets, sink, rb, wb, stream, steps, warmup, repeats) for v in variants]
+        print("[sweep] %s done" % name, file=sys.stderr, flush=True)
+        del sets
+        torch.cuda.empty_cache()
+    print("| chunks/lane | workgroups | order | nt loads | nt stores | " + " | ".join(
+        "%s us (%.1f + %.1f MB)" % (n, r / 1e6, w / 1e6) for n, (r, w) in sizes) + " |")
+    print("|---|---|---|---|---|" + "---|" * len(sizes))
+    for i, v in enumerate(variants):
+        print("| %d | %s | %d | %d | %d | " % (v[0], v[1] or "one step each", v[2], v[3], v[4])
+              + " | ".join("%.2f" % cols[n][i] for n, _ in sizes) + " |")
+    for n, (r, w) in sizes:
+        best = min(range(len(variants)), key=lambda i: cols[n][i])
+        print("best %s: %s %.2f us = %.0f GB/s (%.3f of 8 TB/s)" % (n, variants[best], cols[n][best],
+                                                                  (r + w) / cols[n][best] / 1e3,
+                                                                  (r + w) / cols[n][best] / 1e3 / HBM_PEAK_GBS))
 
 
 def load_traffic_table():
@@ -693,6 +747,8 @@ def main():
     ap.add_argument("--no-headline", action="store_true",
                     help="profiling aid: run only the named configs and print their results without the headline line")
     ap.add_argument("--hot-only", action="store_true", help="profiling aid: one buffer set, no rotation")
+    ap.add_argument("--stream-sweep", action="store_true",
+                    help="time every variant of the no-work kernel on three configurations' byte counts and print a table")
     args = ap.parse_args()
     SETTLE_US = max(0.0, args.settle_us)
     if args.gpus != 1:
@@ -708,6 +764,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
+    if args.stream_sweep:
+        stream_sweep(dev, stream, args.steps, args.warmup, min(3, args.repeats))
+        return
     builders = build_cases(set(names), dev)
     traffic = load_traffic_table()
     results = {}
@@ -750,8 +809,9 @@ def main():
         case.sets = []
         torch.cuda.empty_cache()
         if not args.no_ceiling and not name.startswith("stream_"):
-            ceil_us = stream_ceiling(case, dev, stream, args.steps, args.warmup, min(3, args.repeats))
+            ceil_us, ceil_variant = stream_ceiling(case, dev, stream, args.steps, args.warmup, min(3, args.repeats))
             r["stream_us"] = round(ceil_us, 3)
+            r["stream_variant"] = list(ceil_variant)
             r["stream_gb_per_s"] = round(case.algo_bytes / ceil_us / 1e3, 1)
             r["frac_of_stream"] = round(ceil_us / us, 4)
             torch.cuda.empty_cache()

@@ -59,6 +59,15 @@ const char* fq_last_error(void);
  * counters are calibrated on it. */
 int fq_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink, int nontemporal,
                  void* stream);
+/* The same kernel in its variants (no counterpart in the reference either): chunks_per_lane = 16-byte
+ * chunks in flight per lane (4, 8 or 16); workgroups = how many to launch (0: one step of
+ * 256 * chunks_per_lane chunks per workgroup, else each walks several); order 0 = interleaved steps,
+ * 1 = one contiguous run per workgroup, 2 = the same with one contiguous eighth of the buffers per XCD;
+ * nt_loads / nt_stores put the streaming hint on loads / stores.  fq_stream_rw is
+ * (4, 16384, 0, nontemporal, nontemporal).  The measured ceiling is the fastest variant. */
+int fq_stream_rw_variant(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,
+                         int chunks_per_lane, int64_t workgroups, int order, int nt_loads, int nt_stores,
+                         void* stream);
 
 /* triton_blockwise_quant, linghe/quant/block.py:129-170.
  * x bf16 [M,N], N % 128 == 0.  q [M,N], s [N/128, M], qt [N, M], st [ceil(M/128), N]. */

@@ -27,6 +27,7 @@ _F = ctypes.c_float
 # name -> argtypes, exactly the declarations of include/fq_api.h
 SIGNATURES = {
     "fq_stream_rw": [_P, _L, _P, _L, _P, _I, _P],
+    "fq_stream_rw_variant": [_P, _L, _P, _L, _P, _I, _L, _I, _I, _I, _P],
     "fq_blockwise_quant": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_blockwise_quant": [_P, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_pad_permute_quant": [_P, _P, _I, _I, _L, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _P],

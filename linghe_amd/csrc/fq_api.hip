@@ -63,17 +63,29 @@ int fq_version(void) { return 100; }
 
 const char* fq_last_error(void) { return g_err; }
 
-int fq_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink, int nontemporal,
-                 void* stream) {
-  const char* fn = "fq_stream_rw";
+int fq_stream_rw_variant(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,
+                         int chunks_per_lane, int64_t workgroups, int order, int nt_loads, int nt_stores,
+                         void* stream) {
+  const char* fn = "fq_stream_rw_variant";
   FQ_REQUIRE(read_bytes >= 0 && write_bytes >= 0 && read_bytes % 16 == 0 && write_bytes % 16 == 0, FQ_ERR_SHAPE,
              "%s: byte counts must be non-negative multiples of 16", fn);
   FQ_REQUIRE((read_bytes == 0 || (src && aligned16(src))) && (write_bytes == 0 || (dst && aligned16(dst))) && sink &&
                  aligned16(sink),
              FQ_ERR_ARG, "%s: NULL or misaligned pointer", fn);
-  return check_launch(fq::launch_stream_rw(src, read_bytes, dst, write_bytes, sink, nontemporal != 0,
-                                           (hipStream_t)stream),
+  FQ_REQUIRE(chunks_per_lane == 4 || chunks_per_lane == 8 || chunks_per_lane == 16, FQ_ERR_ARG,
+             "%s: chunks_per_lane must be 4, 8 or 16", fn);
+  FQ_REQUIRE(order >= 0 && order <= 2 && workgroups >= 0 && workgroups <= (1 << 24), FQ_ERR_ARG,
+             "%s: order must be 0, 1 or 2 and workgroups 0 .. 2^24", fn);
+  return check_launch(fq::launch_stream_rw(src, read_bytes, dst, write_bytes, sink, chunks_per_lane, workgroups, order,
+                                           nt_loads != 0, nt_stores != 0, (hipStream_t)stream),
                       fn);
+}
+
+int fq_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink, int nontemporal,
+                 void* stream) {
+  // the plain form: 4 chunks per lane, at most 64 workgroups per CU, interleaved steps
+  return fq_stream_rw_variant(src, read_bytes, dst, write_bytes, sink, 4, 256 * 64, 0, nontemporal, nontemporal,
+                              stream);
 }
 
 int fq_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t N,

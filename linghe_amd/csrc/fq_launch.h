@@ -64,8 +64,10 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
                                        int64_t M, int K, int N, float eps, int round_scale, int kind,
                                        hipStream_t stream);
 
-// measurement aid: read read_bytes from src, write write_bytes to dst (both multiples of 16), no arithmetic
+// measurement aid: read read_bytes from src, write write_bytes to dst (both multiples of 16), no arithmetic;
+// chunks_per_lane 4 / 8 / 16, workgroups (0: one step each), order 0 / 1 / 2, hint on loads / stores
 hipError_t launch_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,
-                            int nontemporal, hipStream_t stream);
+                            int chunks_per_lane, int64_t workgroups, int order, int nt_loads, int nt_stores,
+                            hipStream_t stream);
 
 }  // namespace fq

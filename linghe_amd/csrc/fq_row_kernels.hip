@@ -691,12 +691,21 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_lock;
 float* g_scratch_ptr[kMaxDevices] = {};
 
-// device address of `scratch` on the current device
-hipError_t static_scratch_ptr(float** out) {
+// device address of `scratch` on the device that owns `device_ptr` (one of the call's tensors).
+// That device has to be the current one: kernels are launched on the current device, and the
+// symbol lookup answers for it.  A caller whose current device differs gets an error instead of
+// another GPU's array address.
+hipError_t static_scratch_ptr(const void* device_ptr, float** out) {
   int dev = -1;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return err;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  if (device_ptr != nullptr) {
+    hipPointerAttribute_t attr;
+    err = hipPointerGetAttributes(&attr, device_ptr);
+    if (err != hipSuccess) return err;
+    if (attr.device != dev) return hipErrorInvalidDevice;
+  }
   std::lock_guard<std::mutex> hold(g_scratch_lock);
   if (g_scratch_ptr[dev] == nullptr) {
     void* p = nullptr;
@@ -715,7 +724,7 @@ hipError_t launch_rmsnorm_bwd_static(const void* dy, const void* x, const void* 
   const int64_t P = rmsnorm_bwd_partials(M);
   if (P > kStaticPartialRows || n > kStaticPartialWidth) return hipErrorInvalidValue;
   float* part = nullptr;
-  const hipError_t err = static_scratch_ptr(&part);
+  const hipError_t err = static_scratch_ptr(dgamma, &part);
   if (err != hipSuccess) return err;
   return launch_rmsnorm_bwd(dy, x, gamma, rstd, dx, dgamma, part, P, M, n, eps, stream);
 }

@@ -4,51 +4,87 @@
 // configuration (the measured ceiling the kernels are compared with, beside the
 // 8 TB/s of the data sheet); on a known size it calibrates the profiler's
 // FETCH_SIZE / WRITE_SIZE counters.
+//
+// The ceiling is only as good as the best way of moving the bytes, so the kernel comes
+// in variants: 16-byte chunks in flight per lane (4 / 8 / 16), number of workgroups
+// (a multiple of the CU count, or one step per workgroup), the order in which the
+// workgroups of an XCD walk the buffers, and the non-temporal hint on loads and on
+// stores separately.  The benchmark takes the fastest of a short list per byte count.
 #include "fq_device.hpp"
 #include "fq_launch.h"
 
 namespace fq {
 
-template <bool STREAM>
+// UNROLL chunks per lane and step, loads first: UNROLL*16 bytes in flight per lane
+template <int UNROLL, bool NT_LOAD, bool NT_STORE>
 __global__ __launch_bounds__(256) void stream_rw_kernel(const uint4* __restrict__ src, int64_t read_chunks,
                                                         uint4* __restrict__ dst, int64_t write_chunks,
-                                                        uint4* __restrict__ sink) {
-  const int64_t stride = (int64_t)gridDim.x * 256 * 4;
+                                                        uint4* __restrict__ sink, int order) {
   const int64_t most = read_chunks > write_chunks ? read_chunks : write_chunks;
+  constexpr int kStep = 256 * UNROLL;  // chunks per workgroup and step
+  const int64_t steps = (most + kStep - 1) / kStep;
+  const int G = (int)gridDim.x;
+  int wg = (int)blockIdx.x;
+  if (order == 2) {
+    // workgroup i runs on XCD i % 8: give every XCD one contiguous eighth of the steps
+    const int per = (G + 7) >> 3;
+    const int xcd = wg & 7, slot = wg >> 3;
+    const int full = (G & 7) ? (G & 7) : 8;
+    wg = xcd < full ? xcd * per + slot : full * per + (xcd - full) * (per - 1) + slot;
+  }
   uint4 acc = make_uint4(0, 0, 0, 0);
-  // four chunks per thread and step, loads first: 64 bytes in flight per lane, as in the tile kernels
-  for (int64_t base = (int64_t)blockIdx.x * 1024 + threadIdx.x; base < most; base += stride) {
-    uint4 v[4];
+  // order 0: workgroup wg takes the steps wg, wg + G, wg + 2G, ... (at any time the grid works on one
+  // contiguous window of the buffers); order 1 / 2: a contiguous run of per_wg steps per workgroup
+  const int64_t per_wg = (steps + G - 1) / G;
+  int64_t s0 = order == 0 ? wg : (int64_t)wg * per_wg;
+  int64_t s1 = order == 0 ? steps : s0 + per_wg;
+  if (s1 > steps) s1 = steps;
+  const int64_t ds = order == 0 ? G : 1;
+  for (int64_t s = s0; s < s1; s += ds) {
+    const int64_t base = s * kStep + threadIdx.x;
+    uint4 v[UNROLL];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < UNROLL; ++u) {
       const int64_t i = base + u * 256;
       v[u] = make_uint4((uint32_t)i, 0, 0, 0);
-      if (i < read_chunks) v[u] = load16<STREAM>(src + i);
+      if (i < read_chunks) v[u] = load16<NT_LOAD>(src + i);
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < UNROLL; ++u) {
       const int64_t i = base + u * 256;
       acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w;
-      if (i < write_chunks) store16<STREAM>(dst + i, v[u]);
+      if (i < write_chunks) store16<NT_STORE>(dst + i, v[u]);
     }
   }
   // keeps the loads alive when nothing is written; never true for the all-zero or small-integer data of the bench
   if ((acc.x & acc.y & acc.z & acc.w) == 0xffffffffu) *sink = acc;
 }
 
+// chunks_per_lane: 4, 8 or 16.  workgroups: how many to launch; 0 = one step per workgroup.
+// order: 0 interleaved steps, 1 a contiguous run per workgroup, 2 the same with one contiguous eighth per XCD.
 hipError_t launch_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,
-                            int nontemporal, hipStream_t stream) {
+                            int chunks_per_lane, int64_t workgroups, int order, int nt_loads,
+                            int nt_stores, hipStream_t stream) {
   const int64_t rc = read_bytes / 16, wc = write_bytes / 16;
   const int64_t most = rc > wc ? rc : wc;
   if (most == 0) return hipSuccess;
-  int64_t wgs = (most + 1023) / 1024;
-  if (wgs > 256 * 64) wgs = 256 * 64;
-  if (nontemporal)
-    hipLaunchKernelGGL(stream_rw_kernel<true>, dim3((unsigned)wgs), dim3(256), 0, stream, (const uint4*)src, rc,
-                       (uint4*)dst, wc, (uint4*)sink);
-  else
-    hipLaunchKernelGGL(stream_rw_kernel<false>, dim3((unsigned)wgs), dim3(256), 0, stream, (const uint4*)src, rc,
-                       (uint4*)dst, wc, (uint4*)sink);
+  if (chunks_per_lane != 4 && chunks_per_lane != 8 && chunks_per_lane != 16) return hipErrorInvalidValue;
+  if (order < 0 || order > 2) return hipErrorInvalidValue;
+  const int64_t steps = (most + 256 * chunks_per_lane - 1) / (256 * chunks_per_lane);
+  int64_t wgs = workgroups <= 0 || workgroups > steps ? steps : workgroups;
+  if (wgs > (1 << 30)) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)wgs), block(256);
+#define FQ_STREAM(U, L, S)                                                                              \
+  hipLaunchKernelGGL((stream_rw_kernel<U, L, S>), grid, block, 0, stream, (const uint4*)src, rc, (uint4*)dst, wc, \
+                     (uint4*)sink, order)
+#define FQ_STREAM_HINTS(U)                                       \
+  if (nt_loads) { if (nt_stores) FQ_STREAM(U, true, true); else FQ_STREAM(U, true, false); } \
+  else { if (nt_stores) FQ_STREAM(U, false, true); else FQ_STREAM(U, false, false); }
+  if (chunks_per_lane == 4) { FQ_STREAM_HINTS(4) }
+  else if (chunks_per_lane == 8) { FQ_STREAM_HINTS(8) }
+  else { FQ_STREAM_HINTS(16) }
+#undef FQ_STREAM_HINTS
+#undef FQ_STREAM
   return hipGetLastError();
 }
 

@@ -108,6 +108,31 @@ def test_blockwise_quant_dequant_bound(gpu, dtype):
     assert float(q.float().abs().reshape(M, N // 128, 128).amax(2).min()) == fmax
 
 
+@pytest.mark.parametrize("round_scale", [False, True])
+def test_blockwise_quant_negative_zero(gpu, round_scale):
+    """Inputs holding -0.0.  The reference's x / s keeps the sign of a zero (code 0x80); the kernel's
+    two-operation division returns +0 or -0 depending on the sign of the reciprocal's correction term
+    (with power-of-two scales the convert divides itself and keeps the sign).  Both codes decode to
+    zero and the comparison rule counts them as identical; everything else stays bit-exact."""
+    from linghe_amd.quant.block import triton_blockwise_quant
+
+    announce("blockwise_quant with -0.0 inputs", round_scale)
+    M, N = 256, 384
+    x = randn_bf16(gen(14), M, N)
+    x.view(torch.int16)[::3, ::5] = -32768  # bf16 -0.0
+    x[128:, 128:256] = 0.0
+    x.view(torch.int16)[130:140, 128:256] = -32768  # an all-zero group with negative zeros: scale = the floor
+    assert bool((x.view(torch.int16) == -32768).any())
+    ref = O.blockwise_quant(x, round_scale)
+    q, s, qt, st = triton_blockwise_quant(_dev(x, gpu), round_scale=round_scale, output_mode=2)
+    torch.cuda.synchronize()
+    check_quant_pair("blockwise.negzero.row", ref[0], ref[1], q, s, **EXACT)
+    check_quant_pair("blockwise.negzero.col", ref[2], ref[3], qt, st, **EXACT)
+    zero = (x.float() == 0)
+    assert bool(((q.cpu().view(torch.uint8)[zero] & 0x7F) == 0).all())
+    assert bool(((qt.cpu().view(torch.uint8).t()[zero] & 0x7F) == 0).all())
+
+
 @pytest.mark.parametrize("M,N", [(2049, 2048), (64, 128), (1000, 8192 + 128)])
 @pytest.mark.parametrize("round_scale", [False, True])
 def test_group_quant(gpu, M, N, round_scale):

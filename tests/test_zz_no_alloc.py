@@ -48,6 +48,25 @@ def test_rmsnorm_bwd_noalloc_matches_rmsnorm_bwd(gpu):
         assert torch.equal(dx_a.view(torch.int16), dx_b.view(torch.int16))
         assert torch.equal(dg_a.view(torch.int32), dg_b.view(torch.int32))
         assert bool(torch.isfinite(dg_b).all())
+    # the advertised property: the call itself allocates nothing on the device (the driver's count of
+    # free device memory is the same before and after a call whose buffers all exist already)
+    announce("rmsnorm_bwd_noalloc leaves the free-memory count unchanged")
+    g = gen(62)
+    M, n = 2048, 4096
+    x = randn_bf16(g, M, n).to(gpu)
+    dy = randn_bf16(g, M, n).to(gpu)
+    w = gamma_bf16(g, n).to(gpu)
+    dx = torch.empty_like(x)
+    dg = torch.empty((n,), device=gpu, dtype=torch.float32)
+    stream = _lib.stream_of(x)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(gpu)[0]
+    for _ in range(3):
+        rc = L.fq_rmsnorm_bwd_noalloc(dy.data_ptr(), x.data_ptr(), w.data_ptr(), None, dx.data_ptr(), dg.data_ptr(),
+                                      M, n, 1e-6, stream)
+        assert rc == 0, L.fq_last_error()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(gpu)[0] == free_before
     # beyond the fixed array (and the RMSNorm kernels' own limit): refused with a clear error, nothing launched
     rc = L.fq_rmsnorm_bwd_noalloc(None, None, None, None, None, None, 128, 8192 + 128, 1e-6, None)
     assert rc == -2 and L.fq_last_error()
