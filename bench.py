@@ -454,7 +454,7 @@ def build_cases(names, dev):
         add(_n, build=lambda _n=_n: plain_quant_case(_n))
 
     # ---------------------------------------------------------------- next row: RMSNorm + router GEMM + quant
-    def router_case():
+    def router_case(packed=False):
         M, N, K = 8192, 256, 2048
         g = torch.Generator().manual_seed(1104)
         x_cpu = (torch.randn(M, K, generator=g) ** 2).to(torch.bfloat16)
@@ -469,23 +469,31 @@ def build_cases(names, dev):
                      q=torch.empty((M, K), device=dev, dtype=FP8),
                      s=torch.empty((K // 128, M), device=dev, dtype=torch.float32))
             s["ws"] = torch.empty_like(rwd)
-            s["args"] = (_p(s["x"]), _p(nwd), _p(rwd), 0, _p(s["ws"]), _p(s["y"]), _p(s["r"]), _p(s["lg"]), _p(s["q"]), _p(s["s"]),
-                         M, K, N, 1e-6, 0, _lib.FQ_E4M3, stream)
+            if packed:  # the weight re-ordered once, outside the timed calls
+                _lib.check(L.fq_pack_router_weight(_p(rwd), 0, _p(s["ws"]), K, N, stream))
+                s["args"] = (_p(s["x"]), _p(nwd), _p(s["ws"]), 0, _p(s["y"]), _p(s["r"]), _p(s["lg"]), _p(s["q"]),
+                             _p(s["s"]), M, K, N, 1e-6, 0, _lib.FQ_E4M3, stream)
+            else:
+                s["args"] = (_p(s["x"]), _p(nwd), _p(rwd), 0, _p(s["ws"]), _p(s["y"]), _p(s["r"]), _p(s["lg"]),
+                             _p(s["q"]), _p(s["s"]), M, K, N, 1e-6, 0, _lib.FQ_E4M3, stream)
             return s
 
         def launch(s):
-            _lib.check(L.fq_rmsnorm_router_quant_fwd(*s["args"]))
+            _lib.check((L.fq_rmsnorm_router_quant_fwd_packed if packed else L.fq_rmsnorm_router_quant_fwd)(*s["args"]))
 
         def cpu_fn():
             from oracle import fq_oracle as O
             return O.rms_gemm_block_quant_forward(x_cpu, nw_cpu, rw_cpu)
 
-        c = Case("next_router", "triton_rms_norm_fp32_gemm_block_quant_forward(output_mode=0)", [M, N, K],
+        c = Case("next_router_packed" if packed else "next_router",
+                 "triton_rms_norm_fp32_gemm_block_quant_forward(output_mode=0%s)"
+                 % (", packed_route_weight=..." if packed else ""), [M, N, K],
                  configs.rw_router(M, N, K), make_set, launch, cpu_fn)
         c.extra = {"gemm_flops": 2 * M * N * K}
         return c
 
     add("next_router", build=router_case)
+    add("next_router_packed", build=lambda: router_case(True))
 
     # ---------------------------------------------------------------- the no-work stream kernel on a known size
     # (the read / copy rates of the memory system, and the calibration of FETCH_SIZE / WRITE_SIZE)
@@ -728,7 +736,7 @@ def load_traffic_table():
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
        "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
-       "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router",
+       "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed",
        "stream_read", "stream_copy"]
 
 

@@ -173,6 +173,20 @@ int fq_rmsnorm_router_quant_fwd(const void* x, const void* gamma, const void* ro
                                 int64_t M, int64_t K, int64_t N, float eps, int round_scale, int fp8_kind,
                                 void* stream);
 
+/* The two halves of fq_rmsnorm_router_quant_fwd, for callers that keep the re-ordered weight
+ * between weight updates (the reference re-reads route_weight on every call,
+ * linghe/utils/norm.py:736-784; a router weight changes once per optimiser step).
+ * fq_pack_router_weight re-orders route_weight [N,K] (bf16, or fp32 split into two bf16
+ * planes) into `packed` (fq_rmsnorm_router_scratch_bytes() bytes);
+ * fq_rmsnorm_router_quant_fwd_packed is fq_rmsnorm_router_quant_fwd on that buffer, with the
+ * weight_is_fp32 it was packed with.  Results are bit-identical to the one-call form. */
+int fq_pack_router_weight(const void* route_weight, int weight_is_fp32, void* packed, int64_t K, int64_t N,
+                          void* stream);
+int fq_rmsnorm_router_quant_fwd_packed(const void* x, const void* gamma, const void* packed_weight,
+                                       int weight_is_fp32, void* y, float* rstd, float* logits, void* q, float* s,
+                                       int64_t M, int64_t K, int64_t N, float eps, int round_scale, int fp8_kind,
+                                       void* stream);
+
 /* triton_silu_and_block_quant_forward, linghe/utils/silu.py:279-335.
  * x bf16 [M, 2n] (gate | up).  Outputs as fq_blockwise_quant with N = n. */
 int fq_swiglu_quant_fwd(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t n,

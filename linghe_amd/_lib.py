@@ -40,6 +40,8 @@ SIGNATURES = {
     "fq_rmsnorm_bwd_noalloc": [_P, _P, _P, _P, _P, _P, _L, _L, _F, _P],
     "fq_rmsnorm_quant_fwd": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _I, _I, _P],
     "fq_rmsnorm_router_quant_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _I, _P],
+    "fq_pack_router_weight": [_P, _I, _P, _L, _L, _P],
+    "fq_rmsnorm_router_quant_fwd_packed": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _I, _P],
     "fq_swiglu_quant_fwd": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_swiglu_quant_bwd": [_P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_swiglu_quant_fwd": [_P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],

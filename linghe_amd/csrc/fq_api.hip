@@ -313,6 +313,42 @@ int fq_rmsnorm_router_quant_fwd(const void* x, const void* gamma, const void* ro
                       fn);
 }
 
+int fq_pack_router_weight(const void* route_weight, int weight_is_fp32, void* packed, int64_t K, int64_t N,
+                          void* stream) {
+  const char* fn = "fq_pack_router_weight";
+  FQ_REQUIRE(K > 0 && K % 128 == 0 && K <= 8192, FQ_ERR_SHAPE, "%s: K (%lld) must be a multiple of 128 up to 8192", fn,
+             (long long)K);
+  FQ_REQUIRE(N > 0 && N % 128 == 0 && N <= 8192, FQ_ERR_SHAPE,
+             "%s: %lld router outputs (supported: multiples of 128 up to 8192)", fn, (long long)N);
+  FQ_REQUIRE(route_weight && packed && aligned16(route_weight) && aligned16(packed), FQ_ERR_ARG,
+             "%s: NULL or misaligned pointer", fn);
+  return check_launch(fq::launch_pack_router_weight(route_weight, weight_is_fp32 != 0, packed, (int)K, (int)N,
+                                                    (hipStream_t)stream),
+                      fn);
+}
+
+int fq_rmsnorm_router_quant_fwd_packed(const void* x, const void* gamma, const void* packed_weight,
+                                       int weight_is_fp32, void* y, float* rstd, float* logits, void* q, float* s,
+                                       int64_t M, int64_t K, int64_t N, float eps, int round_scale, int fp8_kind,
+                                       void* stream) {
+  const char* fn = "fq_rmsnorm_router_quant_fwd_packed";
+  int rc = check_common(fn, M, K, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_norm_shape(fn, M, K))) return rc;
+  FQ_REQUIRE(M % 32 == 0, FQ_ERR_SHAPE, "%s: M (%lld) is not a multiple of 32", fn, (long long)M);
+  FQ_REQUIRE(N > 0 && N % 128 == 0 && N <= 8192, FQ_ERR_SHAPE,
+             "%s: %lld router outputs (supported: multiples of 128 up to 8192)", fn, (long long)N);
+  if (M == 0) return FQ_OK;
+  FQ_REQUIRE(x && gamma && packed_weight && y && rstd && logits && q && s, FQ_ERR_ARG, "%s: NULL pointer", fn);
+  FQ_REQUIRE(aligned16(x) && aligned16(gamma) && aligned16(packed_weight) && aligned16(y), FQ_ERR_ARG,
+             "%s: misaligned pointer", fn);
+  FQ_REQUIRE((reinterpret_cast<uintptr_t>(q) & 7u) == 0, FQ_ERR_ARG, "%s: q must be 8-byte aligned", fn);
+  return check_launch(fq::launch_rmsnorm_router_quant_packed(x, gamma, packed_weight, weight_is_fp32 != 0, y, rstd,
+                                                             logits, q, s, M, (int)K, (int)N, eps, round_scale,
+                                                             fp8_kind, (hipStream_t)stream),
+                      fn);
+}
+
 int fq_swiglu_quant_fwd(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int64_t n,
                         int round_scale, int output_mode, int fp8_kind, void* stream) {
   const char* fn = "fq_swiglu_quant_fwd";

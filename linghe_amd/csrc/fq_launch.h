@@ -64,6 +64,14 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
                                        int64_t M, int K, int N, float eps, int round_scale, int kind,
                                        hipStream_t stream);
 
+// the two halves of launch_rmsnorm_router_quant: re-order the weight (once per weight update),
+// run on the re-ordered weight
+hipError_t launch_pack_router_weight(const void* wr, int weight_fp32, void* wpacked, int K, int N, hipStream_t stream);
+hipError_t launch_rmsnorm_router_quant_packed(const void* x, const void* gamma, const void* wpacked,
+                                              int weight_fp32, void* y, float* rstd, float* logits, void* q,
+                                              float* s, int64_t M, int K, int N, float eps, int round_scale,
+                                              int kind, hipStream_t stream);
+
 // measurement aid: read read_bytes from src, write write_bytes to dst (both multiples of 16), no arithmetic;
 // chunks_per_lane 4 / 8 / 16, workgroups (0: one step each), order 0 / 1 / 2, hint on loads / stores
 hipError_t launch_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,

@@ -468,10 +468,32 @@ int64_t rmsnorm_router_scratch_bytes(int K, int N, int weight_fp32) {
   return (int64_t)N * K * (weight_fp32 ? 4 : 2);  // the bf16 planes of W in operand order
 }
 
-hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, int weight_fp32,
-                                       void* wpacked, void* y, float* rstd, float* logits, void* q, float* s,
-                                       int64_t M, int K, int N, float eps, int round_scale, int kind,
-                                       hipStream_t stream) {
+// W [N, K] (bf16 or fp32) -> the operand order of the main kernels, chunk by chunk of 512 virtual
+// columns.  A router weight changes once per optimiser step, so a caller can pack it once and
+// reuse the result for every forward in between.
+hipError_t launch_pack_router_weight(const void* wr, int weight_fp32, void* wpacked, int K, int N,
+                                     hipStream_t stream) {
+  const int vcols = weight_fp32 ? 2 * N : N;  // virtual bf16 columns
+  for (int v0 = 0; v0 < vcols; v0 += 512) {
+    const int vtiles = (vcols - v0 < 512 ? vcols - v0 : 512) / 32;
+    uint4* chunk_w = (uint4*)wpacked + (int64_t)v0 * K / 8;
+    const int64_t pieces = (int64_t)vtiles * 32 * K / 8;
+    const dim3 pgrid((unsigned)((pieces + 255) / 256));
+    if (weight_fp32)
+      hipLaunchKernelGGL(pack_router_weight_kernel<true>, pgrid, dim3(256), 0, stream, wr, chunk_w, K, v0, vtiles);
+    else
+      hipLaunchKernelGGL(pack_router_weight_kernel<false>, pgrid, dim3(256), 0, stream, wr, chunk_w, K, v0, vtiles);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+// the main kernels on a weight already in operand order
+hipError_t launch_rmsnorm_router_quant_packed(const void* x, const void* gamma, const void* wpacked,
+                                              int weight_fp32, void* y, float* rstd, float* logits, void* q,
+                                              float* s, int64_t M, int K, int N, float eps, int round_scale,
+                                              int kind, hipStream_t stream) {
   if (M == 0) return hipSuccess;
   const int vcols = weight_fp32 ? 2 * N : N;  // virtual bf16 columns
   const dim3 grid((unsigned)(M / kRouterRows));
@@ -517,15 +539,7 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
   for (int v0 = 0; v0 < vcols; v0 += 512) {
     const int vtiles = (vcols - v0 < 512 ? vcols - v0 : 512) / 32;
     const bool first = v0 == 0;
-    uint4* chunk_w = (uint4*)wpacked + (int64_t)v0 * K / 8;
-    const int64_t pieces = (int64_t)vtiles * 32 * K / 8;
-    const dim3 pgrid((unsigned)((pieces + 255) / 256));
-    if (weight_fp32)
-      hipLaunchKernelGGL(pack_router_weight_kernel<true>, pgrid, dim3(256), 0, stream, wr, chunk_w, K, v0, vtiles);
-    else
-      hipLaunchKernelGGL(pack_router_weight_kernel<false>, pgrid, dim3(256), 0, stream, wr, chunk_w, K, v0, vtiles);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    const uint4* chunk_w = (const uint4*)wpacked + (int64_t)v0 * K / 8;
     const LogitsOut lout{logits, N, weight_fp32 ? v0 / 2 : v0};
     if (weight_fp32) {
       constexpr bool PAIRV = true;
@@ -534,7 +548,7 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
       constexpr bool PAIRV = false;
       FQ_ROUTER_TILES()
     }
-    e = hipGetLastError();
+    const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
 #undef FQ_ROUTER_TILES
@@ -543,6 +557,17 @@ hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const v
 #undef FQ_ROUTER_STREAMED
 #undef FQ_ROUTER_ARGS
   return hipSuccess;
+}
+
+hipError_t launch_rmsnorm_router_quant(const void* x, const void* gamma, const void* wr, int weight_fp32,
+                                       void* wpacked, void* y, float* rstd, float* logits, void* q, float* s,
+                                       int64_t M, int K, int N, float eps, int round_scale, int kind,
+                                       hipStream_t stream) {
+  if (M == 0) return hipSuccess;
+  const hipError_t e = launch_pack_router_weight(wr, weight_fp32, wpacked, K, N, stream);
+  if (e != hipSuccess) return e;
+  return launch_rmsnorm_router_quant_packed(x, gamma, wpacked, weight_fp32, y, rstd, logits, q, s, M, K, N, eps,
+                                            round_scale, kind, stream);
 }
 
 }  // namespace fq

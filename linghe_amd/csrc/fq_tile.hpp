@@ -38,14 +38,41 @@ struct TileOut {
   float* st;        // column scales:        st[st_off + c]
   int64_t st_off;
   int rows_valid;   // rows i < rows_valid exist (1..128)
+  // A PACKED partial tile: the workgroup covers 2^kc_shift neighbouring column blocks of a row
+  // block with at most 128 >> kc_shift rows (see SubTile); the offsets above are those of the
+  // first column block, the next ones lie s_cb / t_cb elements further (q and st: 128).
+  int kc_shift;     // 0 (one column block, up to 128 rows), 1 or 2
+  int n_sub;        // column blocks that exist (1 .. 1 << kc_shift)
+  int64_t s_cb;     // distance between the row scales of neighbouring column blocks
+  int64_t t_cb;     // distance between their transposed codes (128 * t_ld)
 };
+
+// Which part of a (possibly packed) tile a thread works on.  With kc_shift = k the row groups of
+// the workgroup are split into 2^k sub-tiles of 128 >> k rows, one per column block; a sub-tile is
+// a whole number of waves, so `sub` is the same in every lane of a wave.
+template <int RPT>
+struct SubTile {
+  int sub;   // column block inside the workgroup's run (wave-uniform)
+  int rgl;   // row group inside the sub-tile: rows rgl*RPT .. rgl*RPT+RPT-1
+  int ws;    // wave inside the sub-tile
+};
+template <int RPT>
+__device__ __forceinline__ SubTile<RPT> sub_tile(int kc_shift) {
+  const int rg = threadIdx.x >> 4;
+  const int rgs = (kGroup / RPT) >> kc_shift;  // row groups per sub-tile
+  SubTile<RPT> t;
+  t.sub = __builtin_amdgcn_readfirstlane(rg / rgs);
+  t.rgl = rg & (rgs - 1);
+  t.ws = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6) & ((rgs >> 2) - 1));
+  return t;
+}
 
 // NV: value tiles quantised together by one workgroup (2 in the SwiGLU backward: dx1, dx2)
 template <int RPT, int NV = 1>
 struct alignas(16) TileShared {
   uint8_t t[NV][kGroup * kGroup];                        // transposed codes, 16-byte chunks XOR-swizzled
   float colmax[NV][TileShape<RPT>::kWaves][kGroup];       // per-wave column amax
-  float2 cdiv[NV][kGroup];                                // per column what the quantiser keeps per scale (Quantum)
+  float2 cdiv[NV][NV == 1 ? 4 : 1][kGroup];               // per column (and sub-tile of a packed tile) what the quantiser keeps per scale (Quantum)
   float2 rdiv[NV][kGroup];                                // per row    the same
 };
 
@@ -108,12 +135,16 @@ __device__ __forceinline__ uint32_t pick_dword(uint32_t d0, uint32_t d1, uint32_
 // Called by the 8 threads ch = 0..7 that share the row: thread ch owns source
 // bytes [16 ch, 16 ch + 16); a chunk cut by the end of the row leaves as at most
 // one 8-, 4-, 2- and 1-byte store.
+// In a packed tile the 128 bytes of an LDS row hold the rows of several sub-tiles one after
+// the other: the thread reads chunk `ch` of the LDS row and writes it as chunk `chd` of its
+// sub-tile's transposed row (ch == chd in an unpacked tile).
 template <bool STREAM>
-__device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uint8_t* dst_row, int len, int ch) {
-  const int rem = len - 16 * ch;
+__device__ __forceinline__ void store_t_row(const uint8_t* lds_row, int swz, uint8_t* dst_row, int len, int ch,
+                                            int chd) {
+  const int rem = len - 16 * chd;
   if (rem <= 0) return;
   const uint4 v = *(const uint4*)(lds_row + ((ch ^ swz) * 16));
-  uint8_t* dst = dst_row + 16 * ch;
+  uint8_t* dst = dst_row + 16 * chd;
   if (rem >= 16) {
     store16_any<STREAM>(dst, v);
     return;
@@ -144,12 +175,19 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
   const int cg = tid & 15;
   const int rg = tid >> 4;
   const int rows_valid = o[0].rows_valid;
+  // packed partial tiles: this wave's column block (sub) and its rows inside it; a full tile
+  // is one sub-tile and the compiler sees the constants
+  const int kc_shift = (FULL || NV > 1) ? 0 : o[0].kc_shift;  // several value tiles are never packed
+  SubTile<RPT> sl;
+  if constexpr (FULL) { sl.sub = 0; sl.rgl = rg; sl.ws = wave; }
+  else sl = sub_tile<RPT>(kc_shift);
+  const int rgl = sl.rgl;
 
   // A wave owns 4*RPT consecutive rows.  In a partial tile the waves whose rows all
-  // lie beyond the last stored row have nothing to quantise: their values are
-  // zero, their row-wise outputs do not exist and their bytes of the transposed
-  // tile are never stored, so they only keep the barriers company.
-  const bool live = FULL || wave * (4 * RPT) < rows_valid;
+  // lie beyond the last stored row (or whose column block does not exist) have nothing
+  // to quantise: their values are zero, their row-wise outputs do not exist and their
+  // bytes of the transposed tile are never stored, so they only keep the barriers company.
+  const bool live = FULL || (sl.ws * (4 * RPT) < rows_valid && sl.sub < o[0].n_sub);
 
   // LEAN: the four output bases, which are the same in every lane, are moved to scalar
   // registers, so that each store is "scalar base + 32-bit lane offset" (a tile spans
@@ -167,6 +205,12 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
     t_base[t] = o[t].qt + o[t].t_off;
     s_base[t] = o[t].s + o[t].s_off;
     st_base[t] = o[t].st + o[t].st_off;
+    if constexpr (!FULL) {  // this wave's column block of a packed tile
+      q_base[t] += sl.sub * kGroup;
+      s_base[t] += sl.sub * o[t].s_cb;
+      // t_base / st_base stay those of the first column block: the threads that store the
+      // transposed rows and the column scales are not the ones that computed them
+    }
     if constexpr (LEAN) {
       q_base[t] = (uint8_t*)uniform64((int64_t)q_base[t]);
       t_base[t] = (uint8_t*)uniform64((int64_t)t_base[t]);
@@ -199,8 +243,8 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
       if (cg < RPT) {
         const float sc = make_scale<KIND, ROUND>(mine);
         const Quantum<ROUND> d = make_quantum<ROUND>(sc);
-        const int i = rg * RPT + cg;
-        sh.rdiv[t][i] = make_float2(d.a, d.b);
+        const int i = rgl * RPT + cg;
+        sh.rdiv[t][rg * RPT + cg] = make_float2(d.a, d.b);
         if (FULL || i < rows_valid) store_f32(s_base[t] + (uint32_t)i, sc);  // a wave writes 4*RPT consecutive floats
       }
     }
@@ -214,7 +258,7 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
         const float2 sr = sh.rdiv[t][rg * RPT + s];
         const Quantum<ROUND> d{sr.x, sr.y};
         const uint2 pk = quantize8<KIND, ROUND>(v[t][s], d);
-        const int i = rg * RPT + s;
+        const int i = rgl * RPT + s;
         if (FULL || i < rows_valid) store8<(NT & 2) != 0>(q_base[t] + ((uint32_t)i * q_ld + (uint32_t)cg * 8u), pk);
       }
     }
@@ -261,18 +305,32 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
       }
     }
     __syncthreads();
-    if (tid < NV * kGroup) {  // thread (t, c): the scale of column c of tile t
-      const int t = tid / kGroup, c = tid % kGroup;
-      float m = sh.colmax[t][0][c];
+    if constexpr (FULL || NV > 1) {
+      if (tid < NV * kGroup) {  // thread (t, c): the scale of column c of tile t
+        const int t = tid / kGroup, c = tid % kGroup;
+        float m = sh.colmax[t][0][c];
 #pragma unroll
-      for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[t][w][c]);
-      const float sc = make_scale<KIND, ROUND>(m);
-      const Quantum<ROUND> d = make_quantum<ROUND>(sc);
-      sh.cdiv[t][c] = make_float2(d.a, d.b);
-      float* dst = st_base[0];
+        for (int w = 1; w < Shape::kWaves; ++w) m = fmaxf(m, sh.colmax[t][w][c]);
+        const float sc = make_scale<KIND, ROUND>(m);
+        const Quantum<ROUND> d = make_quantum<ROUND>(sc);
+        sh.cdiv[t][0][c] = make_float2(d.a, d.b);
+        float* dst = st_base[0];
 #pragma unroll
-      for (int u = 1; u < NV; ++u) dst = (t == u) ? st_base[u] : dst;
-      store_f32(dst + (uint32_t)c, sc);
+        for (int u = 1; u < NV; ++u) dst = (t == u) ? st_base[u] : dst;
+        store_f32(dst + (uint32_t)c, sc);
+      }
+    } else {
+      // thread (sb, c): the scale of column c of sub-tile sb, over that sub-tile's waves
+      const int wps = Shape::kWaves >> kc_shift;
+      for (int idx = tid; idx < o[0].n_sub * kGroup; idx += Shape::kThreads) {
+        const int sb = idx / kGroup, c = idx % kGroup;
+        float m = 0.f;
+        for (int w = 0; w < wps; ++w) m = fmaxf(m, sh.colmax[0][sb * wps + w][c]);
+        const float sc = make_scale<KIND, ROUND>(m);
+        const Quantum<ROUND> d = make_quantum<ROUND>(sc);
+        sh.cdiv[0][sb][c] = make_float2(d.a, d.b);
+        store_f32(st_base[0] + (uint32_t)(sb * kGroup + c), sc);
+      }
     }
     __syncthreads();
     if (live) {
@@ -280,7 +338,7 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
       for (int t = 0; t < NV; ++t) {
         Quantum<ROUND> cd[8];
         {
-          const float4* src = (const float4*)&sh.cdiv[t][cg * 8];
+          const float4* src = (const float4*)&sh.cdiv[t][FULL ? 0 : sl.sub][cg * 8];
 #pragma unroll
           for (int h = 0; h < 4; ++h) {
             const float4 a = src[h];
@@ -320,7 +378,13 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
           const uint4 val = *(const uint4*)(sh.t[t] + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
           store16_any<(NT & 1) != 0>(t_base[t] + ((uint32_t)c * t_ld + (uint32_t)ch * 16u), val);
         } else {
-          store_t_row<(NT & 1) != 0>(sh.t[t] + c * kGroup, (c >> 3) & 7, t_base[t] + (uint32_t)c * t_ld, rows_valid, ch);
+          // LDS row c holds, one after the other, the rows of column c of every sub-tile
+          const int cps = 8 >> kc_shift;  // 16-byte chunks per sub-tile
+          const int sb = ch / cps;
+          const int len = sb < o[t].n_sub ? rows_valid : 0;
+          store_t_row<(NT & 1) != 0>(sh.t[t] + c * kGroup, (c >> 3) & 7,
+                                     t_base[t] + ((int64_t)sb * o[t].t_cb + (int64_t)((uint32_t)c * t_ld)), len, ch,
+                                     ch & (cps - 1));
         }
       }
     }
@@ -354,6 +418,8 @@ struct ExpertTile {
   int count;            // rows of this expert
   int pcount;           // rows of its region in the outputs: count rounded up to a multiple of `pad`
   int rb;               // 128-row block inside the expert
+  int cb;               // first 128-column block of the workgroup
+  int kc_shift;         // the workgroup covers 1 << kc_shift column blocks (packed partial tile), 0 = one
   int64_t row_start;    // first global row of the expert's region (sum of the pcount before it)
   int64_t tblock_start; // sum over previous experts of ceil(count/128)
 };
@@ -374,17 +440,27 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
   return v;
 }
 
-// Which expert owns the global 128-row block `blk` (blocks are numbered expert
-// after expert, ceil(count/128) per expert)?  Computed from the device-side
-// counts by a prefix scan that EVERY WAVE runs for itself, 64 experts per step with
-// the loads of up to sixteen steps in flight together: no LDS, no barrier, and every
-// thread of the workgroup ends with the same answer.  (A workgroup-wide scan
-// with three barriers cost 13 % of the batched SwiGLU forward.)  An out-of-range
-// blk (host and device counts disagree) yields expert = -1.
+// How many neighbouring column blocks one workgroup takes in the LAST row block of an expert
+// whose (padded) count leaves `last` rows there: a block of at most 64 (32) rows leaves half
+// (three quarters) of a 128-row workgroup without rows, so the idle waves take the next column
+// block(s) of the same rows instead: 1 << shift column blocks of 128 >> shift rows each.
+// Column maxima stay per column, row maxima per row and column block: nothing else changes.
+__device__ __forceinline__ int pack_shift(int last_rows) { return last_rows <= 32 ? 2 : last_rows <= 64 ? 1 : 0; }
+
+// Which tile does workgroup `wg` of a per-expert launch own?  Workgroups are numbered expert
+// after expert; an expert with nbk = ceil(count/128) row blocks takes (nbk - 1) * ncb workgroups
+// for its full row blocks (row block after row block, ncb column blocks each) and
+// ceil(ncb / kc) for its last one, kc = 1 << pack_shift(rows of the last block).  Computed from
+// the device-side counts by a prefix scan that EVERY WAVE runs for itself, 64 experts per step
+// with the loads of up to sixteen steps in flight together: no LDS, no barrier, and every
+// thread of the workgroup ends with the same answer.  (A workgroup-wide scan with three
+// barriers cost 13 % of the batched SwiGLU forward.)  A workgroup beyond the last tile (the
+// launch is sized for one workgroup per 128 x 128 tile, packing needs fewer) or counts that
+// disagree with the host's yield expert = -1.
 // pad > 1: every expert's region starts at a multiple of pad rows (the reference's
 // permute-and-pad layout, pad = 16); 128 is a multiple of pad, so the number of
 // 128-row blocks of an expert does not change.
-__device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int is_i64, int n_experts, int blk,
+__device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int is_i64, int n_experts, int wg, int ncb,
                                                        int pad = 1) {
   const int lane = threadIdx.x & 63;
   ExpertTile t;
@@ -392,9 +468,11 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
   t.count = 0;
   t.pcount = 0;
   t.rb = 0;
+  t.cb = 0;
+  t.kc_shift = 0;
   t.row_start = 0;
   t.tblock_start = 0;
-  int run_rows = 0, run_blocks = 0;
+  int run_rows = 0, run_blocks = 0, run_wgs = 0;
   // the counts of up to 1024 experts (16 steps) are fetched together: one memory round
   // trip however many steps the scan then takes
   constexpr int kSteps = 16;
@@ -417,23 +495,38 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
         const int c = cs[k];
         const int pc = (c + pad - 1) & -pad;  // pad is a power of two (1 or 16)
         const int nb = (c + kGroup - 1) / kGroup;
+        const int shift = pack_shift(pc - (nb - 1) * kGroup);
+        const int kc = 1 << shift;
+        const int nw = nb > 0 ? (nb - 1) * ncb + ((ncb + kc - 1) >> shift) : 0;
         const int rows = wave_inclusive_scan(pc);
         const int blocks = wave_inclusive_scan(nb);
-        const int excl_blocks = run_blocks + blocks - nb;
-        const bool hit = nb > 0 && blk >= excl_blocks && blk < excl_blocks + nb;
+        const int wgs = wave_inclusive_scan(nw);
+        const int excl_wgs = run_wgs + wgs - nw;
+        const bool hit = nw > 0 && wg >= excl_wgs && wg < excl_wgs + nw;
         const unsigned long long mask = __builtin_amdgcn_ballot_w64(hit);
         if (mask != 0) {
           const int src = __builtin_ctzll(mask);
           t.expert = base + src;
           t.count = __builtin_amdgcn_readlane(c, src);
           t.pcount = __builtin_amdgcn_readlane(pc, src);
-          t.tblock_start = __builtin_amdgcn_readlane(excl_blocks, src);
-          t.rb = blk - t.tblock_start;
+          t.tblock_start = run_blocks + __builtin_amdgcn_readlane(blocks - nb, src);
           t.row_start = (int64_t)(run_rows + __builtin_amdgcn_readlane(rows - pc, src));
+          const int local = wg - __builtin_amdgcn_readlane(excl_wgs, src);
+          const int nbe = __builtin_amdgcn_readlane(nb, src);
+          const int full = (nbe - 1) * ncb;  // workgroups of the expert's full row blocks
+          if (local < full) {
+            t.rb = local / ncb;
+            t.cb = local - t.rb * ncb;
+          } else {
+            t.rb = nbe - 1;
+            t.kc_shift = __builtin_amdgcn_readlane(shift, src);
+            t.cb = (local - full) << t.kc_shift;
+          }
           return t;
         }
         run_rows += __builtin_amdgcn_readlane(rows, 63);
         run_blocks += __builtin_amdgcn_readlane(blocks, 63);
+        run_wgs += __builtin_amdgcn_readlane(wgs, 63);
       }
     }
   }

@@ -12,7 +12,9 @@ struct TileGeom {
   int64_t row0;      // first global row of the tile
   int rows_valid;    // rows that exist in the input (and in the outputs unless padded)
   int rows_store;    // rows written to the outputs (>= rows_valid; the extra ones hold zeros)
-  int cb;            // 128-column block of the input
+  int cb;            // (first) 128-column block of the input
+  int kc_shift;      // packed partial tile: 1 << kc_shift column blocks of at most 128 >> kc_shift rows
+  int n_sub;         // of which exist (the run may end at the matrix edge)
   int64_t s_base, s_stride;
   int64_t t_base, t_stride;
   int64_t st_row;
@@ -29,28 +31,41 @@ struct BatchArgs {
 
 // out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
 // backward's dx1|dx2)
-// remap: workgroup i runs on XCD i % 8; give every XCD one contiguous eighth of the
-// tiles instead of every eighth tile.  Which order of the tiles the memory system likes
+// remap: workgroup i runs on XCD i % 8; 1 = give every XCD one contiguous eighth of the
+// tiles instead of every eighth tile, 2 = give it every eighth row block (see below).  Which order of the tiles the memory system likes
 // better depends on the kernel and the shape (measured: the RMSNorm tile kernel 4-18 %
 // faster with it at 16384 x 7168 and slower below ~2000 tiles or with narrow rows, the
 // per-expert SwiGLU backward 5 % faster; gather+pad+quant 18 % slower, the blockwise
 // quantisers 5-9 %, the forward SwiGLU kernels 2-4 %), so the caller decides.
 template <bool BATCHED>
 __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out_w, const BatchArgs& b,
-                                                 bool remap = false) {
+                                                 int remap = 0) {
   TileGeom g;
   int id = blockIdx.x;
-  if (remap) {  // workgroup-uniform
+  if (remap == 1) {  // workgroup-uniform
     const int G = (int)gridDim.x;
     const int per = (G + 7) >> 3;
     const int xcd = id & 7, slot = id >> 3;
     // the first (G % 8, or 8) XCDs hold `per` tiles, the others one fewer
     const int full = (G & 7) ? (G & 7) : 8;
     id = xcd < full ? xcd * per + slot : full * per + (xcd - full) * (per - 1) + slot;
+  } else if (remap == 2) {
+    // runs of ncb consecutive tiles (one row block) stay on one XCD, the runs go round the XCDs:
+    // the neighbours in memory share an L2, and work that ends early in the numbering (a launch
+    // sized for more workgroups than there are tiles) is spread over all XCDs
+    const int G = (int)gridDim.x;
+    const int span = 8 * ncb;
+    if (id < G - G % span) {
+      const int xcd = id & 7, slot = id >> 3;
+      const int run = slot / ncb;
+      id = (run * 8 + xcd) * ncb + (slot - run * ncb);
+    }
   }
-  const int rbk = id / ncb;
-  g.cb = id - rbk * ncb;
+  g.kc_shift = 0;
+  g.n_sub = 1;
   if constexpr (!BATCHED) {
+    const int rbk = id / ncb;
+    g.cb = id - rbk * ncb;
     g.row0 = (int64_t)rbk * kGroup;
     const int64_t left = M - g.row0;
     g.rows_valid = left < kGroup ? (int)left : kGroup;
@@ -63,10 +78,14 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
     g.expert = 0;
     g.valid = left > 0;
   } else {
-    const ExpertTile et = find_expert_tile(b.counts, b.counts_i64, b.n_experts, rbk, b.pad > 1 ? b.pad : 1);
+    const ExpertTile et = find_expert_tile(b.counts, b.counts_i64, b.n_experts, id, ncb, b.pad > 1 ? b.pad : 1);
     // the lookup's answer is the same in every lane: keep it in scalar registers
     const int expert = uniform32(et.expert), count = uniform32(et.count), rb = uniform32(et.rb);
     const int pcount = uniform32(et.pcount);
+    g.cb = uniform32(et.cb);
+    g.kc_shift = uniform32(et.kc_shift);
+    const int cbs_left = ncb - g.cb;
+    g.n_sub = cbs_left < (1 << g.kc_shift) ? cbs_left : (1 << g.kc_shift);
     const int64_t row_start = uniform64(et.row_start), tblock_start = uniform64(et.tblock_start);
     g.valid = expert >= 0;
     g.expert = expert;
@@ -106,16 +125,22 @@ __device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g,
   o.st = p.st;
   o.st_off = g.st_row * out_w + (int64_t)ocb * kGroup;
   o.rows_valid = g.rows_store;
+  o.kc_shift = g.kc_shift;
+  o.n_sub = g.n_sub;
+  o.s_cb = g.s_stride;
+  o.t_cb = (int64_t)kGroup * g.t_stride;
   return o;
 }
 
 // RPT rows x 8 bf16 columns of a row-major matrix; rows >= rows_valid read as 0
 // STREAM: loads carry the non-temporal hint (the tile is not read again).
-// SCALAR: the tile base, the same in every lane, is moved to scalar registers
+// SCALAR: the tile base, the same in every lane of a wave, is moved to scalar registers
+// rgl: the thread's row group (rows rgl*RPT ..): threadIdx.x >> 4 in an unpacked tile, the row
+// group inside the wave's sub-tile in a packed one (then base points at that sub-tile's columns)
 template <int RPT, bool STREAM = false, bool SCALAR = true>
-__device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
+__device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT],
+                                          int rgl) {
   const int cg = threadIdx.x & 15;
-  const int rg = threadIdx.x >> 4;
   // a tile spans at most 128 rows of at most 2^24 bytes (the widest input the entry
   // points accept), so lane offsets fit 32 bits
   const uint8_t* b = (const uint8_t*)base;
@@ -124,7 +149,7 @@ __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int 
     b = (const uint8_t*)uniform64((int64_t)b);
     pitch = (uint32_t)uniform32((int)pitch);
   }
-  const uint32_t off0 = (uint32_t)(rg * RPT) * pitch + (uint32_t)cg * 16u;
+  const uint32_t off0 = (uint32_t)(rgl * RPT) * pitch + (uint32_t)cg * 16u;
   if (rows_valid == kGroup) {  // workgroup-uniform: no per-row masks
 #pragma unroll
     for (int s = 0; s < RPT; ++s) raw[s] = load16<STREAM>(b + (off0 + (uint32_t)s * pitch));
@@ -132,9 +157,29 @@ __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int 
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
       raw[s] = make_uint4(0, 0, 0, 0);
-      if (rg * RPT + s < rows_valid) raw[s] = load16<STREAM>(b + (off0 + (uint32_t)s * pitch));
+      if (rgl * RPT + s < rows_valid) raw[s] = load16<STREAM>(b + (off0 + (uint32_t)s * pitch));
     }
   }
+}
+template <int RPT, bool STREAM = false, bool SCALAR = true>
+__device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
+  load_rows<RPT, STREAM, SCALAR>(base, ld, rows_valid, raw, (int)(threadIdx.x >> 4));
+}
+
+// The part of a (possibly packed) tile this thread's wave works on, and how many of its rows exist
+template <int RPT>
+struct TilePart {
+  SubTile<RPT> sl;
+  int rows;  // rows of this wave's sub-tile that exist (0: the column block lies beyond the matrix)
+  int cb;    // its 128-column block
+};
+template <int RPT>
+__device__ __forceinline__ TilePart<RPT> tile_part(const TileGeom& g) {
+  TilePart<RPT> p;
+  p.sl = sub_tile<RPT>(g.kc_shift);
+  p.rows = p.sl.sub < g.n_sub ? g.rows_valid : 0;
+  p.cb = g.cb + p.sl.sub;
+  return p;
 }
 
 #define FQ_DISPATCH_BOOL(flag, NAME, ...) \

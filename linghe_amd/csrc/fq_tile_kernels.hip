@@ -98,6 +98,12 @@
 // when its division took three operations per element; with the current two it is level
 // at 16384 x 7168 (110.5 us either way, 58.9 / 58.5 us with the statistic given) and
 // 2 % behind at 8192 x 2048 (18.3 / 18.0 us), so it runs with 4.
+#ifndef FQ_BWD_REMAP
+#define FQ_BWD_REMAP 0
+#endif
+#ifndef FQ_FWD_REMAP
+#define FQ_FWD_REMAP 0
+#endif
 #ifndef FQ_BWD_PIN
 #define FQ_BWD_PIN 1
 #endif
@@ -123,7 +129,8 @@ __global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __
   constexpr bool LDNT = (BATCHED ? FQ_LDNT_BLOCKWISE_B : FQ_LDNT_BLOCKWISE) != 0;
   constexpr int NT = BATCHED ? FQ_NT_BLOCKWISE_B : FQ_NT_BLOCKWISE;
   constexpr bool LEAN = BATCHED || FQ_LEAN_BLOCKWISE != 0;
-  load_rows<RPT, LDNT, LEAN>(x + g.row0 * N + (int64_t)g.cb * kGroup, N, g.rows_valid, raw);
+  const TilePart<RPT> tp = tile_part<RPT>(g);
+  load_rows<RPT, LDNT, LEAN>(x + g.row0 * N + (int64_t)tp.cb * kGroup, N, tp.rows, raw, tp.sl.rgl);
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
@@ -148,7 +155,8 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
   const TileGeom g = resolve_tile<true>(M, N / kGroup, N, batch);
   if (!g.valid) return;
   const int cg = threadIdx.x & 15;
-  const int rg = threadIdx.x >> 4;
+  const TilePart<RPT> tp = tile_part<RPT>(g);
+  const int rg = tp.sl.rgl;
   // the 8 source rows of this thread: two 16-byte loads (regions start at multiples of 16 rows)
   int src[RPT];
 #pragma unroll
@@ -160,12 +168,12 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
     src[4] = b.x; src[5] = b.y; src[6] = b.z; src[7] = b.w;
   }
   uint4 raw[RPT];
-  const uint16_t* col = x + (int64_t)g.cb * kGroup + cg * 8;
+  const uint16_t* col = x + (int64_t)tp.cb * kGroup + cg * 8;
 #pragma unroll
   for (int s = 0; s < RPT; ++s) {
     raw[s] = make_uint4(0, 0, 0, 0);
     // rows of the padding, and indices that do not name a source row, read as zero
-    if (rg * RPT + s < g.rows_valid && (uint32_t)src[s] < (uint64_t)src_rows)
+    if (rg * RPT + s < tp.rows && (uint32_t)src[s] < (uint64_t)src_rows)
       raw[s] = load16<FQ_LDNT_PERMUTE != 0>(col + (int64_t)src[s] * N);
   }
   if (probs != nullptr && g.cb == 0 && threadIdx.x < kGroup) {
@@ -199,22 +207,23 @@ __global__ __launch_bounds__(2048 / FQ_RPT_FWD) void silu_quant_fwd_kernel(const
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {
   constexpr int RPT = FQ_RPT_FWD;
   __shared__ TileShared<RPT> sh;
-  const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch);
+  const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch, BATCHED ? FQ_FWD_REMAP : 0);
   if (!g.valid) return;
   const int64_t ld = 2 * (int64_t)n;
   uint4 r1[RPT], r2[RPT];
   const uint16_t* p = x + g.row0 * ld + (int64_t)g.cb * kGroup;
   constexpr bool LDNT = (BATCHED ? FQ_LDNT_SILU_FWD_B : FQ_LDNT_SILU_FWD) != 0;
   constexpr int NT = MODE == 0 ? FQ_NT_SILU_FWD_M0 : MODE == 1 ? FQ_NT_SILU_FWD_M1 : BATCHED ? FQ_NT_SILU_FWD_B : FQ_NT_SILU_FWD;
-  load_rows<RPT, LDNT>(p, ld, g.rows_valid, r1);
-  load_rows<RPT, LDNT>(p + n, ld, g.rows_valid, r2);
-  const int rg = threadIdx.x >> 4;
+  const TilePart<RPT> tp = tile_part<RPT>(g);
+  load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, ld, tp.rows, r1, tp.sl.rgl);
+  load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, ld, tp.rows, r2, tp.sl.rgl);
+  const int rg = tp.sl.rgl;
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s)
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[s][j] = 0.f;
-  if ((threadIdx.x >> 6) * (4 * RPT) < g.rows_valid) {  // waves beyond the last row of a partial tile keep zeros
+  if (tp.sl.ws * (4 * RPT) < tp.rows) {  // waves beyond the last row of a partial tile keep zeros
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
       float a[8], b[8];
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(2048 / FQ_RPT_FWD) void silu_quant_fwd_kernel(const
       float w = 1.0f;
       if constexpr (WEIGHTED) {
         const int i = rg * RPT + s;
-        w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
+        w = (i < tp.rows) ? load_weight(weight, g.row0 + i) : 0.f;
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -250,24 +259,25 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   constexpr int RPT = 4;
   const int nb = n / kGroup;
   const int64_t N = 2 * (int64_t)n;
-  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch, BATCHED);  // the per-expert form takes the XCD remap
+  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch, BATCHED ? FQ_BWD_REMAP : 0);  // the per-expert form takes an XCD remap
   if (!g.valid) return;
   uint4 r1[RPT], r2[RPT], rgd[RPT];
   const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
   constexpr bool LDNT = (BATCHED ? FQ_LDNT_SILU_BWD_B : FQ_LDNT_SILU_BWD) != 0;
   constexpr int NT = BATCHED ? FQ_NT_SILU_BWD_B : FQ_NT_SILU_BWD;
-  load_rows<RPT, LDNT>(p, N, g.rows_valid, r1);
-  load_rows<RPT, LDNT>(p + n, N, g.rows_valid, r2);
-  load_rows<RPT, LDNT>(gr + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, rgd);
+  const TilePart<RPT> tp = tile_part<RPT>(g);
+  load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, N, tp.rows, r1, tp.sl.rgl);
+  load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, N, tp.rows, r2, tp.sl.rgl);
+  load_rows<RPT, LDNT>(gr + g.row0 * n + (int64_t)tp.cb * kGroup, n, tp.rows, rgd, tp.sl.rgl);
   const int cg = threadIdx.x & 15;
-  const int rg = threadIdx.x >> 4;
+  const int rg = tp.sl.rgl;
   float d[2][RPT][8];  // dx1, dx2
   float my_dw = 0.f;
 #pragma unroll
   for (int s = 0; s < RPT; ++s)
 #pragma unroll
     for (int j = 0; j < 8; ++j) d[0][s][j] = d[1][s][j] = 0.f;
-  if ((threadIdx.x >> 6) * (4 * RPT) < g.rows_valid) {  // waves beyond the last row of a partial tile keep zeros
+  if (tp.sl.ws * (4 * RPT) < tp.rows) {  // waves beyond the last row of a partial tile keep zeros
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
 #if FQ_BWD_PIN
@@ -290,7 +300,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
       unpack8(rgd[s], go);
       float w = 1.0f;
       const int i = rg * RPT + s;
-      if constexpr (BATCHED) w = (i < g.rows_valid) ? load_weight(weight, g.row0 + i) : 0.f;
+      if constexpr (BATCHED) w = (i < tp.rows) ? load_weight(weight, g.row0 + i) : 0.f;
       float dw = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -314,7 +324,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   if constexpr (BATCHED) {
     if (cg < RPT) {
       const int i = rg * RPT + cg;
-      if (i < g.rows_valid) dw_part[(g.row0 + i) * nb + g.cb] = my_dw;
+      if (i < tp.rows) dw_part[(g.row0 + i) * nb + tp.cb] = my_dw;
     }
   }
   if constexpr (!BATCHED) {
@@ -359,7 +369,7 @@ __global__ __launch_bounds__(2048 / FQ_RPT_RMS) void rmsnorm_quant_tile_kernel(c
   constexpr int RPT = FQ_RPT_RMS;
   __shared__ TileShared<RPT> sh;
   BatchArgs none{nullptr, 0, 0};
-  const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none, remap != 0);
+  const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none, remap);
   if (!g.valid) return;
   uint4 raw[RPT];
   load_rows<RPT, FQ_LDNT_RMSNORM != 0>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);

@@ -154,6 +154,27 @@ def triton_rms_norm_and_block_quant_forward(
     return out, scale, rms, transpose_output, transpose_scale
 
 
+def pack_route_weight(route_weight: torch.Tensor) -> torch.Tensor:
+    """The router weight [N, K] (bf16 or fp32) in the operand order the RMSNorm + router GEMM
+    kernels read it in, as a uint8 tensor to pass as `packed_route_weight=` of
+    triton_rms_norm_fp32_gemm_block_quant_forward.  No counterpart in the reference, which
+    re-reads route_weight on every call: re-pack after every update of the weight."""
+    assert route_weight.is_contiguous() and route_weight.dim() == 2
+    if route_weight.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"route_weight must be bfloat16 or float32, got {route_weight.dtype}")
+    if not route_weight.is_cuda:
+        raise RuntimeError("route_weight must live on the GPU: the HIP kernels are the only implementation")
+    N, K = route_weight.size()
+    assert K % 128 == 0 and N % 128 == 0
+    w_fp32 = int(route_weight.dtype == torch.float32)
+    packed = torch.empty(int(_lib.lib.fq_rmsnorm_router_scratch_bytes(K, N, w_fp32)), dtype=torch.uint8,
+                         device=route_weight.device)
+    with _lib.on_device(route_weight.device):
+        _lib.check(_lib.lib.fq_pack_router_weight(_lib.ptr(route_weight), w_fp32, _lib.ptr(packed), K, N,
+                                                  _lib.stream_of(route_weight)))
+    return packed
+
+
 def triton_rms_norm_fp32_gemm_block_quant_forward(
     x: torch.Tensor,
     norm_weight: torch.Tensor,
@@ -162,6 +183,8 @@ def triton_rms_norm_fp32_gemm_block_quant_forward(
     eps: float = 1e-6,
     output_mode: int = 0,
     round_scale=False,
+    *,
+    packed_route_weight: Optional[torch.Tensor] = None,
 ):
     """
     y = rms_norm(x)
@@ -175,6 +198,10 @@ def triton_rms_norm_fp32_gemm_block_quant_forward(
         output_mode: 0 or 1
             0: only output non-transpose quantizatino tensor (and y, rms, logits)
             1: only output transposed quantizatino tensor (rms must be given)
+        packed_route_weight: (keyword-only addition) the result of pack_route_weight(route_weight).
+            The kernels read the router weight in matrix-core operand order; without this
+            argument it is re-ordered on every call, with it the caller re-orders once per
+            weight update.  Results are identical.
 
     Returns:
         - y: rms normed tensor
@@ -213,13 +240,21 @@ def triton_rms_norm_fp32_gemm_block_quant_forward(
             if not route_weight.is_cuda:
                 raise RuntimeError("route_weight must live on the GPU: the HIP kernels are the only implementation")
             w_fp32 = int(route_weight.dtype == torch.float32)
-            # route_weight re-ordered for the matrix cores (an fp32 weight as two bf16 planes)
-            scratch = torch.empty(int(_lib.lib.fq_rmsnorm_router_scratch_bytes(K, N, w_fp32)), dtype=torch.uint8,
-                                  device=device)
-            _lib.check(_lib.lib.fq_rmsnorm_router_quant_fwd(
-                _lib.ptr(x), _lib.ptr(norm_weight), _lib.ptr(route_weight), w_fp32, _lib.ptr(scratch), _lib.ptr(y), _lib.ptr(rms),
-                _lib.ptr(logits), _lib.ptr(x_q), _lib.ptr(x_s), M, K, N, float(eps), int(bool(round_scale)),
-                _lib.FQ_E4M3, _lib.stream_of(x)))
+            need = int(_lib.lib.fq_rmsnorm_router_scratch_bytes(K, N, w_fp32))
+            if packed_route_weight is not None:
+                assert packed_route_weight.is_cuda and packed_route_weight.dtype == torch.uint8
+                assert packed_route_weight.numel() == need and packed_route_weight.is_contiguous()
+                _lib.check(_lib.lib.fq_rmsnorm_router_quant_fwd_packed(
+                    _lib.ptr(x), _lib.ptr(norm_weight), _lib.ptr(packed_route_weight), w_fp32, _lib.ptr(y),
+                    _lib.ptr(rms), _lib.ptr(logits), _lib.ptr(x_q), _lib.ptr(x_s), M, K, N, float(eps),
+                    int(bool(round_scale)), _lib.FQ_E4M3, _lib.stream_of(x)))
+            else:
+                # route_weight re-ordered for the matrix cores (an fp32 weight as two bf16 planes)
+                scratch = torch.empty(need, dtype=torch.uint8, device=device)
+                _lib.check(_lib.lib.fq_rmsnorm_router_quant_fwd(
+                    _lib.ptr(x), _lib.ptr(norm_weight), _lib.ptr(route_weight), w_fp32, _lib.ptr(scratch),
+                    _lib.ptr(y), _lib.ptr(rms), _lib.ptr(logits), _lib.ptr(x_q), _lib.ptr(x_s), M, K, N, float(eps),
+                    int(bool(round_scale)), _lib.FQ_E4M3, _lib.stream_of(x)))
         else:
             _lib.check(_lib.lib.fq_rmsnorm_quant_fwd(
                 _lib.ptr(x), _lib.ptr(norm_weight), None, None, _lib.ptr(rms), _lib.ptr(xt_q), _lib.ptr(xt_s),

@@ -165,7 +165,8 @@ def test_entry_points_keep_reference_signatures(ref):
     positional = [p.name for p in sig.parameters.values() if p.kind == p.POSITIONAL_OR_KEYWORD]
     assert positional == params, (ref, positional)
     extras = [p.name for p in sig.parameters.values() if p.kind == p.KEYWORD_ONLY]
-    assert set(extras) <= {"fp8_dtype"}
+    # additions are keyword-only: the FP8 format, and the caller-packed router weight
+    assert set(extras) <= {"fp8_dtype", "packed_route_weight"}
 
 
 def test_host_asserts_fire_on_cpu_tensors():

@@ -449,7 +449,9 @@ def test_block_quant(gpu, M, N, round_scale):
     (256, 256, 1536, torch.float32),
     # more than 512 (virtual) columns: one launch per chunk of 512
     (256, 1024, 2048, torch.bfloat16), (128, 640, 1536, torch.bfloat16), (128, 384, 2048, torch.float32),
-    (128, 1024, 1024, torch.float32)])
+    (128, 1024, 1024, torch.float32),
+    # the widest router the entry point accepts: 16 launches (bf16) / 32 virtual-column chunks (fp32)
+    (128, 8192, 256, torch.bfloat16), (128, 8192, 128, torch.float32)])
 @pytest.mark.parametrize("round_scale", [False, True])
 def test_rms_norm_fp32_gemm_block_quant(gpu, M, N, K, wdtype, round_scale):
     """reference tests/test_norm.py:251-287 (x = randn**2, weights randn; the reference's
@@ -485,6 +487,15 @@ def test_rms_norm_fp32_gemm_block_quant(gpu, M, N, K, wdtype, round_scale):
     print(f"[parity] router.logits: max abs err {err:.3e}, sum|y||w| max {scale:.3e}", flush=True)
     assert err <= 2e-5 * scale
     torch.testing.assert_close(logits.cpu(), ref[2], rtol=1e-3, atol=0.1)
+    # the weight re-ordered once by the caller: bit-identical results
+    from linghe_amd.utils.norm import pack_route_weight
+    packed = pack_route_weight(rwd)
+    yp, rmsp, logitsp, qp, sp, _, _ = fn(xd, nwd, rwd, round_scale=round_scale, output_mode=0,
+                                         packed_route_weight=packed)
+    torch.cuda.synchronize()
+    assert torch.equal(logitsp.cpu(), logits.cpu()) and torch.equal(rmsp.cpu(), rms.cpu())
+    assert torch.equal(yp.cpu().view(torch.int16), y.cpu().view(torch.int16))
+    assert torch.equal(qp.cpu().view(torch.uint8), q.cpu().view(torch.uint8)) and torch.equal(sp.cpu(), s.cpu())
     # output_mode 1: the transposed copy from the saved statistic
     _, rms1, _, _, _, qt, st = fn(xd, nwd, rwd, rms=rms, round_scale=round_scale, output_mode=1)
     torch.cuda.synchronize()
