@@ -1,0 +1,96 @@
+// Tuning policy of the kernels: cache hints, rows per thread, tile order.  Every value here
+// was chosen by measurement on MI355X with cold inputs (buffers rotated beyond the memory-side
+// cache); results are identical whatever the values.  One table for the whole library.
+//
+// A sweep build may replace the table: compile with -DFQ_POLICY_HEADER='"my_policy.hpp"', a
+// header that defines fq::Policy with the same members.
+#pragma once
+
+#ifdef FQ_POLICY_HEADER
+#include FQ_POLICY_HEADER
+#else
+namespace fq {
+
+struct Policy {
+  // ---- which code stores carry the non-temporal hint (bit 0: transposed codes, bit 1: row-wise
+  // codes).  With it the outputs do not displace inputs from L2 and the memory-side cache:
+  // gather+pad+quant 75 -> 55 us, RMSNorm+quant after the statistic pass 25 -> 21 us
+  // (8192 x 2048) and 146 -> 122 us (16384 x 7168).  The SwiGLU backward is 3-7 % slower when its
+  // transposed stores carry it; the plain blockwise quantiser takes none (13.2 us at 8192 x 2048
+  // against 14.2-16.1 with any), its per-expert form the transposed stores only (31.5 us against
+  // 39.2 without, 32.7 with the row-wise codes only and 36.3 with both); the RMSNorm tile kernel
+  // with the statistic given (transposed output only, x read once: nothing to protect) none
+  // (16384 x 7168: 66.6 -> 59.5 us).  Transposed rows that do not start on 16-byte boundaries
+  // (M or a per-expert count that is not a multiple of 16) are where the hint on the transposed
+  // stores costs most: the SwiGLU forward takes 100 instead of 70 us at 16300 x 3584 with it (and
+  // gains 3 % at 8192 x 2048), so it keeps the hint on the row-wise codes only; the RMSNorm tile
+  // kernel gains 18 % from it on aligned rows and loses 8 % on unaligned ones.
+  static constexpr int kStoreHintBlockwise = 0;
+  static constexpr int kStoreHintBlockwiseBatched = 1;
+  static constexpr int kStoreHintPermute = 3;
+  static constexpr int kStoreHintSiluFwd = 2;        // both layouts, single matrix
+  static constexpr int kStoreHintSiluFwdRows = 2;    // row-wise layout only
+  static constexpr int kStoreHintSiluFwdCols = 1;    // transposed layout only
+  static constexpr int kStoreHintSiluFwdBatched = 2;
+  static constexpr int kStoreHintSiluBwd = 2;
+  static constexpr int kStoreHintSiluBwdBatched = 2;
+  static constexpr int kStoreHintRmsnorm = 3;        // both layouts (x is read again: protect it)
+  static constexpr int kStoreHintRmsnormCols = 0;    // transposed output only, statistic given
+
+  // ---- the bulk loads carry the hint (3-5 % on the SwiGLU kernels and the RMSNorm tile kernel,
+  // 12 % on the plain blockwise quantiser, 6 % on its per-expert form; the gathered rows, which
+  // several experts read, are 27 % slower with it)
+  static constexpr bool kLoadHintBlockwise = true;
+  static constexpr bool kLoadHintBlockwiseBatched = true;
+  static constexpr bool kLoadHintPermute = false;
+  static constexpr bool kLoadHintSiluFwd = true;
+  static constexpr bool kLoadHintSiluFwdBatched = true;
+  static constexpr bool kLoadHintSiluBwd = true;
+  static constexpr bool kLoadHintSiluBwdBatched = true;
+  static constexpr bool kLoadHintRmsnorm = true;
+
+  // ---- the lean form of the quantiser and of the tile loads (scalar bases, paired
+  // column-maximum reduction; every other tile kernel uses it, -3 to -9 %) in the PLAIN
+  // blockwise quantiser, which is 7 % slower with it (48 -> 51 us at 65536 x 1024); the
+  // per-expert form takes it (Zipf counts: 60.6 -> 57.9 us)
+  static constexpr bool kLeanBlockwise = false;
+
+  // ---- rows per thread (workgroup = 2048 / rows threads).  8 rows per thread spread the
+  // per-thread overhead over twice the elements, 4 rows per thread put twice the waves on a CU.
+  // The SwiGLU forward needs 135 registers with 8 and loses 5-9 %.  The RMSNorm tile kernel
+  // measured 3-4 % ahead with 8 (93 registers, five 256-thread workgroups per CU) when its
+  // division took three operations per element; with the current two it is level at
+  // 16384 x 7168 (110.5 us either way, 58.9 / 58.5 us with the statistic given) and 2 % behind at
+  // 8192 x 2048 (18.3 / 18.0 us), so it runs with 4.
+  static constexpr int kRowsPerThreadSiluFwd = 4;
+  static constexpr int kRowsPerThreadRmsnorm = 4;
+
+  // ---- the per-expert SwiGLU backward widens row s of its packed inputs after row s-1 is done
+  // (fence_values): 136 -> 122 registers, no spill under its cap of 128
+  static constexpr bool kPinBwdRowsBatched = true;
+  static constexpr bool kPinBwdRows = false;
+
+  // ---- tile order across the XCDs (resolve_tile: 0 grid order, 1 one contiguous eighth of the
+  // tiles per XCD, 2 every eighth row block per XCD).  With partial tiles packed the per-expert
+  // SwiGLU backward runs 87.5 us in grid order, 89.3 with order 2 and 95.3 with order 1 (its
+  // launch is sized for one workgroup per 128 x 128 tile, so the workgroups that find no tile
+  // all land on the last XCDs); the forward is level.
+  static constexpr int kTileOrderSiluBwdBatched = 0;
+  static constexpr int kTileOrderSiluFwdBatched = 0;
+
+  // ---- row kernels: the outputs are written once (-3 to -7 % with the hint on the RMSNorm
+  // backward, the bf16 SwiGLU rows and the 128x128 block quantiser); the loads of rows that a
+  // kernel reads once carry it too; RMSNorm + row-wise quant gives every XCD one contiguous
+  // eighth of the rows (13.0 -> 12.4 us at 8192 x 2048)
+  static constexpr bool kStoreHintRows = true;
+  static constexpr bool kLoadHintRows = true;
+  static constexpr bool kXcdContiguousRowQuant = true;
+
+  // ---- router kernels: hint on the stores of y and the codes, and on the loads of x in the
+  // register-resident kernel
+  static constexpr bool kStoreHintRouter = true;
+  static constexpr bool kLoadHintRouter = true;
+};
+
+}  // namespace fq
+#endif

@@ -37,17 +37,11 @@
 // (v/4)*8 + (l/32)*4 + v%4 in register v.
 #include "fq_device.hpp"
 #include "fq_launch.h"
+#include "fq_policy.hpp"
 
 namespace fq {
 
-// cache policy (see load16/store16): FQ_ROUTER_NT puts the non-temporal hint on the
-// stores of y and the codes, FQ_ROUTER_LDNT on the loads of x in the resident kernel
-#ifndef FQ_ROUTER_NT
-#define FQ_ROUTER_NT 1
-#endif
-#ifndef FQ_ROUTER_LDNT
-#define FQ_ROUTER_LDNT 1
-#endif
+// cache hints: fq_policy.hpp
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx16_t __attribute__((ext_vector_type(16)));
@@ -240,9 +234,9 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
       if constexpr (SIDE) {
         m = row16_max(m);
         const float sc = make_scale<KIND, ROUND>(m);
-        store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, hi);
+        store16<Policy::kStoreHintRouter>(yrow + (int64_t)u * K + kb * kGroup, hi);
         const uint2 pk = quantize8<KIND, ROUND>(yv, make_quantum<ROUND>(sc));
-        store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
+        store8<Policy::kStoreHintRouter>(qrow + (int64_t)u * K + kb * kGroup, pk);
         if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
       }
     }
@@ -345,7 +339,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
   auto w_piece = [&](int kb, int t, int j) { return wlane[((int64_t)kb * WAVES * NT + t) * 8 * 64 + j * 64]; };
   auto fetch_x = [&](int kb, uint4 (&xk)[RPT]) {
 #pragma unroll
-    for (int u = 0; u < RPT; ++u) xk[u] = load16<FQ_ROUTER_LDNT != 0>(xrow + (int64_t)u * K + kb * kGroup);
+    for (int u = 0; u < RPT; ++u) xk[u] = load16<Policy::kLoadHintRouter>(xrow + (int64_t)u * K + kb * kGroup);
   };
 #pragma unroll
   for (int d = 0; d < kWAhead; ++d)
@@ -455,9 +449,9 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
         }
         m = row16_max(m);
         const float sc = make_scale<KIND, ROUND>(m);
-        store16<FQ_ROUTER_NT != 0>(yrow + (int64_t)u * K + kb * kGroup, pack8_bf16(yv));
+        store16<Policy::kStoreHintRouter>(yrow + (int64_t)u * K + kb * kGroup, pack8_bf16(yv));
         const uint2 pk = quantize8<KIND, ROUND>(yv, make_quantum<ROUND>(sc));
-        store8<FQ_ROUTER_NT != 0>(qrow + (int64_t)u * K + kb * kGroup, pk);
+        store8<Policy::kStoreHintRouter>(qrow + (int64_t)u * K + kb * kGroup, pk);
         if (cg == 0) s[(int64_t)kb * M + row0 + RPT * rg + u] = sc;
       }
     }

@@ -15,26 +15,14 @@
 
 #include "fq_device.hpp"
 #include "fq_launch.h"
+#include "fq_policy.hpp"
 
 namespace fq {
 
-// Cache policy (see load16/store16): the outputs of these kernels are written once
-// (-3 to -7 % with the hint on the RMSNorm backward, the bf16 SwiGLU rows and the
-// 128x128 block quantiser); FQ_ROW_LDNT puts the hint on the loads of rows that the
-// kernel reads once.
-#ifndef FQ_FWD_REMAP
-#define FQ_FWD_REMAP 1
-#endif
-#ifndef FQ_NT_ROWS
-#define FQ_NT_ROWS 1
-#endif
-#ifndef FQ_ROW_LDNT
-#define FQ_ROW_LDNT 1
-#endif
-
-__device__ __forceinline__ void st16(void* p, const uint4& v) { store16<FQ_NT_ROWS != 0>(p, v); }
-__device__ __forceinline__ void st8(void* p, const uint2& v) { store8<FQ_NT_ROWS != 0>(p, v); }
-__device__ __forceinline__ uint4 ld16(const void* p) { return load16<FQ_ROW_LDNT != 0>(p); }
+// cache hints of the row kernels: fq_policy.hpp
+__device__ __forceinline__ void st16(void* p, const uint4& v) { store16<Policy::kStoreHintRows>(p, v); }
+__device__ __forceinline__ void st8(void* p, const uint2& v) { store8<Policy::kStoreHintRows>(p, v); }
+__device__ __forceinline__ uint4 ld16(const void* p) { return load16<Policy::kLoadHintRows>(p); }
 
 
 template <int T>
@@ -169,7 +157,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
   // workgroup i runs on XCD i % 8, and every XCD takes one contiguous eighth of the
   // indices in the quantising form (3-7 % faster; the bf16 form is 8-20 % slower with it)
   int64_t r0 = blockIdx.x;
-  if constexpr (OUT == 1 && FQ_FWD_REMAP != 0) {
+  if constexpr (OUT == 1 && Policy::kXcdContiguousRowQuant) {
     const int Gi = (int)gridDim.x;
     const int per = (Gi + 7) >> 3;
     const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
@@ -211,7 +199,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
         if (c * 8 < n) {
           // codes of wide rows (the four-waves-per-row form) go out with ordinary stores: 71 -> 67.6 us at
           // 16384 x 7168; narrow rows keep the hint (12.5 against 13.0 us at 8192 x 2048)
-          store8<FQ_NT_ROWS != 0 && T == 64>((uint8_t*)out + row * n + c * 8, pk);
+          store8<Policy::kStoreHintRows && T == 64>((uint8_t*)out + row * n + c * 8, pk);
           if ((c & 15) == 0) scale[(int64_t)(c >> 4) * M + row] = sc;
         }
       }
@@ -224,19 +212,19 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
     uint4 buf[NCHUNK];
     int parity = 0;
     for (int64_t row = r0; row < r1; row += G) {
-      load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + row * n, n, buf);
+      load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + row * n, n, buf);
       process(buf, row, parity);
       parity ^= 1;
     }
     return;
   }
   uint4 bufA[NCHUNK], bufB[NCHUNK];
-  load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + r0 * n, n, bufA);
+  load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + r0 * n, n, bufA);
   for (int64_t row = r0; row < r1; row += 2 * G) {
-    if (row + G < r1) load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + (row + G) * n, n, bufB);
+    if (row + G < r1) load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + (row + G) * n, n, bufB);
     process(bufA, row, 0);
     if (row + G < r1) {
-      if (row + 2 * G < r1) load_row_clamped<T, NCHUNK, FQ_ROW_LDNT != 0>(x + (row + 2 * G) * n, n, bufA);
+      if (row + 2 * G < r1) load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + (row + 2 * G) * n, n, bufA);
       process(bufB, row + G, 1);
     }
   }
@@ -332,8 +320,8 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
     uint4 rx[NCHUNK], rg[NCHUNK];
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
-      rx[k] = load16<FQ_ROW_LDNT != 0>(x + row * n + cidx[k] * 8);
-      rg[k] = load16<FQ_ROW_LDNT != 0>(dy + row * n + cidx[k] * 8);
+      rx[k] = load16<Policy::kLoadHintRows>(x + row * n + cidx[k] * 8);
+      rg[k] = load16<Policy::kLoadHintRows>(dy + row * n + cidx[k] * 8);
     }
     double ss = 0.0;
     float dot = 0.f;

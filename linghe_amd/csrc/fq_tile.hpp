@@ -22,6 +22,16 @@ struct TileShape {
   static constexpr int kRowGroups = kGroup / RPT;
   static constexpr int kThreads = 16 * kRowGroups;
   static constexpr int kWaves = kThreads / 64;
+  // LDS tile of transposed codes: one row of kPitch bytes per column, its 128 code bytes as eight
+  // 16-byte chunks of which chunk k sits at position k ^ swizzle(column group).  With 4 rows per
+  // thread the 4-byte column writes of a wave pair up column groups cg and cg + 8 on one bank; a
+  // pitch of 144 bytes with the swizzle on cg >> 1, which spreads a wave's 64 writes over 64
+  // distinct banks, was measured and is not used: more LDS instructions (the compiler no longer
+  // pairs the writes), 10 % MORE conflict cycles in total (688128 against 622592 per dispatch at
+  // 8192 x 2048) and the same kernel times within 1 % - most of the counted cycles are the
+  // natural extra cycles of the 16-byte-per-lane reads, not the writes.
+  static constexpr int kPitch = kGroup;
+  __device__ static __forceinline__ int swizzle(int cg) { return cg & 7; }
 };
 
 // where the four outputs of one tile go (element offsets; see the layout
@@ -70,7 +80,7 @@ __device__ __forceinline__ SubTile<RPT> sub_tile(int kc_shift) {
 // NV: value tiles quantised together by one workgroup (2 in the SwiGLU backward: dx1, dx2)
 template <int RPT, int NV = 1>
 struct alignas(16) TileShared {
-  uint8_t t[NV][kGroup * kGroup];                        // transposed codes, 16-byte chunks XOR-swizzled
+  uint8_t t[NV][kGroup * TileShape<RPT>::kPitch];         // transposed codes, 16-byte chunks XOR-swizzled
   float colmax[NV][TileShape<RPT>::kWaves][kGroup];       // per-wave column amax
   float2 cdiv[NV][NV == 1 ? 4 : 1][kGroup];               // per column (and sub-tile of a packed tile) what the quantiser keeps per scale (Quantum)
   float2 rdiv[NV][kGroup];                                // per row    the same
@@ -336,24 +346,16 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
     if (live) {
 #pragma unroll
       for (int t = 0; t < NV; ++t) {
-        Quantum<ROUND> cd[8];
-        {
-          const float4* src = (const float4*)&sh.cdiv[t][FULL ? 0 : sl.sub][cg * 8];
-#pragma unroll
-          for (int h = 0; h < 4; ++h) {
-            const float4 a = src[h];
-            cd[2 * h].a = a.x; cd[2 * h].b = a.y;
-            cd[2 * h + 1].a = a.z; cd[2 * h + 1].b = a.w;
-          }
-        }
+        const float2* cdp = &sh.cdiv[t][FULL ? 0 : sl.sub][cg * 8];
         // transposed codes -> LDS; byte (c, i) lives at c*128 + ((i>>4) ^ ((c>>3)&7))*16 + (i&15)
         const int i0 = rg * RPT;
-        const int chunk = (i0 >> 4) ^ (cg & 7);
+        const int chunk = (i0 >> 4) ^ Shape::swizzle(cg);
         uint8_t* base = sh.t[t] + chunk * 16 + (i0 & 15);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const Quantum<ROUND> d = cd[j];
-          uint8_t* p = base + (cg * 8 + j) * kGroup;
+          const float2 c2 = cdp[j];
+          const Quantum<ROUND> d{c2.x, c2.y};
+          uint8_t* p = base + (cg * 8 + j) * Shape::kPitch;
           if constexpr (RPT == 8) {
             uint2 pk;
             pk.x = quantize4<KIND, ROUND>(v[t][0][j], v[t][1][j], v[t][2][j], v[t][3][j], d);
@@ -375,14 +377,14 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
       for (int k = 0; k < kGroup / kRowsPerPass; ++k) {
         const int c = (tid >> 3) + k * kRowsPerPass;
         if constexpr (FULL) {
-          const uint4 val = *(const uint4*)(sh.t[t] + c * kGroup + ((ch ^ ((c >> 3) & 7)) * 16));
+          const uint4 val = *(const uint4*)(sh.t[t] + c * Shape::kPitch + ((ch ^ Shape::swizzle(c >> 3)) * 16));
           store16_any<(NT & 1) != 0>(t_base[t] + ((uint32_t)c * t_ld + (uint32_t)ch * 16u), val);
         } else {
           // LDS row c holds, one after the other, the rows of column c of every sub-tile
           const int cps = 8 >> kc_shift;  // 16-byte chunks per sub-tile
           const int sb = ch / cps;
           const int len = sb < o[t].n_sub ? rows_valid : 0;
-          store_t_row<(NT & 1) != 0>(sh.t[t] + c * kGroup, (c >> 3) & 7,
+          store_t_row<(NT & 1) != 0>(sh.t[t] + c * Shape::kPitch, Shape::swizzle(c >> 3),
                                      t_base[t] + ((int64_t)sb * o[t].t_cb + (int64_t)((uint32_t)c * t_ld)), len, ch,
                                      ch & (cps - 1));
         }

@@ -7,112 +7,8 @@
 #include "fq_tile_geom.hpp"
 #include "fq_launch.h"
 
-// Cache policy per kernel, chosen by measurement (cold inputs, MI355X).
-//   FQ_NT_<kernel>: which code stores carry the non-temporal hint (bit 0: transposed
-//   codes, bit 1: row-wise codes).  With it the outputs do not displace inputs from L2
-//   and the memory-side cache: gather+pad+quant 75 -> 55 us, RMSNorm+quant after the
-//   statistic pass 25 -> 21 us (8192 x 2048) and 146 -> 122 us (16384 x 7168).  The
-//   SwiGLU backward is 3-7 % slower when its transposed stores carry it; the plain
-//   blockwise quantiser takes none (13.2 us at 8192 x 2048 against 14.2-16.1 with any), its
-//   per-expert form (suffix _B) the transposed stores only (31.5 us against 39.2 without, 32.7
-//   with the row-wise codes only and 36.3 with both); the RMSNorm tile kernel with the
-//   statistic given (transposed output only, x read once: nothing to protect) none
-//   (16384 x 7168: 66.6 -> 59.5 us).  Transposed rows that do not start
-//   on 16-byte boundaries (M or a per-expert count that is not a multiple of 16) are where
-//   the hint on the transposed stores costs most: the SwiGLU forward takes 100 instead of
-//   70 us at 16300 x 3584 with it (and gains 3 % at 8192 x 2048), so it keeps the hint on
-//   the row-wise codes only; the RMSNorm tile kernel gains 18 % from it on aligned rows
-//   and loses 8 % on unaligned ones.
-//   FQ_LDNT_<kernel>: the bulk loads carry it (3-5 % on the SwiGLU kernels and the
-//   RMSNorm tile kernel, 12 % on the plain blockwise quantiser, 6 % on its per-expert form;
-//   the gathered rows, which several experts read, are 27 % slower with it).
-#ifndef FQ_NT_BLOCKWISE
-#define FQ_NT_BLOCKWISE 0
-#endif
-#ifndef FQ_NT_BLOCKWISE_B
-#define FQ_NT_BLOCKWISE_B 1
-#endif
-#ifndef FQ_NT_PERMUTE
-#define FQ_NT_PERMUTE 3
-#endif
-#ifndef FQ_NT_SILU_FWD
-#define FQ_NT_SILU_FWD 2
-#endif
-#ifndef FQ_NT_SILU_BWD
-#define FQ_NT_SILU_BWD 2
-#endif
-#ifndef FQ_NT_SILU_FWD_M0
-#define FQ_NT_SILU_FWD_M0 2
-#endif
-#ifndef FQ_NT_SILU_FWD_M1
-#define FQ_NT_SILU_FWD_M1 1
-#endif
-#ifndef FQ_NT_SILU_FWD_B
-#define FQ_NT_SILU_FWD_B 2
-#endif
-#ifndef FQ_NT_SILU_BWD_B
-#define FQ_NT_SILU_BWD_B 2
-#endif
-#ifndef FQ_NT_RMSNORM
-#define FQ_NT_RMSNORM 3
-#endif
-// transposed output only (the statistic is given, x is read once: nothing to protect)
-#ifndef FQ_NT_RMSNORM_T
-#define FQ_NT_RMSNORM_T 0
-#endif
-//   FQ_LEAN_BLOCKWISE: the lean form of the quantiser and of the tile loads (scalar
-//   bases, paired column-maximum reduction; every other tile kernel uses it, -3 to -9 %)
-//   in the PLAIN blockwise quantiser, which is 7 % slower with it (48 -> 51 us at
-//   65536 x 1024); the per-expert form takes it (zipf counts: 60.6 -> 57.9 us).
-#ifndef FQ_LEAN_BLOCKWISE
-#define FQ_LEAN_BLOCKWISE 0
-#endif
-#ifndef FQ_LDNT_BLOCKWISE
-#define FQ_LDNT_BLOCKWISE 1
-#endif
-#ifndef FQ_LDNT_BLOCKWISE_B
-#define FQ_LDNT_BLOCKWISE_B 1
-#endif
-#ifndef FQ_LDNT_PERMUTE
-#define FQ_LDNT_PERMUTE 0
-#endif
-#ifndef FQ_LDNT_SILU_FWD
-#define FQ_LDNT_SILU_FWD 1
-#endif
-#ifndef FQ_LDNT_SILU_BWD
-#define FQ_LDNT_SILU_BWD 1
-#endif
-#ifndef FQ_LDNT_SILU_FWD_B
-#define FQ_LDNT_SILU_FWD_B 1
-#endif
-#ifndef FQ_LDNT_SILU_BWD_B
-#define FQ_LDNT_SILU_BWD_B 1
-#endif
-#ifndef FQ_LDNT_RMSNORM
-#define FQ_LDNT_RMSNORM 1
-#endif
-// Rows per thread (workgroup = 2048 / RPT threads).  8 rows per thread spread the
-// per-thread overhead over twice the elements, 4 rows per thread put twice the waves on
-// a CU.  The SwiGLU forward needs 135 registers with 8 and loses 5-9 %.  The RMSNorm tile
-// kernel measured 3-4 % ahead with 8 (93 registers, five 256-thread workgroups per CU)
-// when its division took three operations per element; with the current two it is level
-// at 16384 x 7168 (110.5 us either way, 58.9 / 58.5 us with the statistic given) and
-// 2 % behind at 8192 x 2048 (18.3 / 18.0 us), so it runs with 4.
-#ifndef FQ_BWD_REMAP
-#define FQ_BWD_REMAP 0
-#endif
-#ifndef FQ_FWD_REMAP
-#define FQ_FWD_REMAP 0
-#endif
-#ifndef FQ_BWD_PIN
-#define FQ_BWD_PIN 1
-#endif
-#ifndef FQ_RPT_FWD
-#define FQ_RPT_FWD 4
-#endif
-#ifndef FQ_RPT_RMS
-#define FQ_RPT_RMS 4
-#endif
+#include "fq_policy.hpp"
+
 namespace fq {
 
 // ---------------------------------------------------------------------------
@@ -126,9 +22,9 @@ __global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __
   const TileGeom g = resolve_tile<BATCHED>(M, N / kGroup, N, batch);
   if (!g.valid) return;
   uint4 raw[RPT];
-  constexpr bool LDNT = (BATCHED ? FQ_LDNT_BLOCKWISE_B : FQ_LDNT_BLOCKWISE) != 0;
-  constexpr int NT = BATCHED ? FQ_NT_BLOCKWISE_B : FQ_NT_BLOCKWISE;
-  constexpr bool LEAN = BATCHED || FQ_LEAN_BLOCKWISE != 0;
+  constexpr bool LDNT = BATCHED ? Policy::kLoadHintBlockwiseBatched : Policy::kLoadHintBlockwise;
+  constexpr int NT = BATCHED ? Policy::kStoreHintBlockwiseBatched : Policy::kStoreHintBlockwise;
+  constexpr bool LEAN = BATCHED || Policy::kLeanBlockwise;
   const TilePart<RPT> tp = tile_part<RPT>(g);
   load_rows<RPT, LDNT, LEAN>(x + g.row0 * N + (int64_t)tp.cb * kGroup, N, tp.rows, raw, tp.sl.rgl);
   float v[RPT][8];
@@ -174,7 +70,7 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
     raw[s] = make_uint4(0, 0, 0, 0);
     // rows of the padding, and indices that do not name a source row, read as zero
     if (rg * RPT + s < tp.rows && (uint32_t)src[s] < (uint64_t)src_rows)
-      raw[s] = load16<FQ_LDNT_PERMUTE != 0>(col + (int64_t)src[s] * N);
+      raw[s] = load16<Policy::kLoadHintPermute>(col + (int64_t)src[s] * N);
   }
   if (probs != nullptr && g.cb == 0 && threadIdx.x < kGroup) {
     const int i = threadIdx.x;
@@ -196,24 +92,24 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
-  quantize_tile<KIND, ROUND, 2, RPT, FQ_NT_PERMUTE>(v, make_out(out, g, N, g.cb), sh);
+  quantize_tile<KIND, ROUND, 2, RPT, Policy::kStoreHintPermute>(v, make_out(out, g, N, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
 // SwiGLU forward + quant.  y = (sigmoid(x1)*x1)*x2 [*w_row]   (fp32)
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED>
-__global__ __launch_bounds__(2048 / FQ_RPT_FWD) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
+__global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {
-  constexpr int RPT = FQ_RPT_FWD;
+  constexpr int RPT = Policy::kRowsPerThreadSiluFwd;
   __shared__ TileShared<RPT> sh;
-  const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch, BATCHED ? FQ_FWD_REMAP : 0);
+  const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch, BATCHED ? Policy::kTileOrderSiluFwdBatched : 0);
   if (!g.valid) return;
   const int64_t ld = 2 * (int64_t)n;
   uint4 r1[RPT], r2[RPT];
   const uint16_t* p = x + g.row0 * ld + (int64_t)g.cb * kGroup;
-  constexpr bool LDNT = (BATCHED ? FQ_LDNT_SILU_FWD_B : FQ_LDNT_SILU_FWD) != 0;
-  constexpr int NT = MODE == 0 ? FQ_NT_SILU_FWD_M0 : MODE == 1 ? FQ_NT_SILU_FWD_M1 : BATCHED ? FQ_NT_SILU_FWD_B : FQ_NT_SILU_FWD;
+  constexpr bool LDNT = BATCHED ? Policy::kLoadHintSiluFwdBatched : Policy::kLoadHintSiluFwd;
+  constexpr int NT = MODE == 0 ? Policy::kStoreHintSiluFwdRows : MODE == 1 ? Policy::kStoreHintSiluFwdCols : BATCHED ? Policy::kStoreHintSiluFwdBatched : Policy::kStoreHintSiluFwd;
   const TilePart<RPT> tp = tile_part<RPT>(g);
   load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, ld, tp.rows, r1, tp.sl.rgl);
   load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, ld, tp.rows, r2, tp.sl.rgl);
@@ -259,12 +155,12 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   constexpr int RPT = 4;
   const int nb = n / kGroup;
   const int64_t N = 2 * (int64_t)n;
-  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch, BATCHED ? FQ_BWD_REMAP : 0);  // the per-expert form takes an XCD remap
+  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch, BATCHED ? Policy::kTileOrderSiluBwdBatched : 0);  // the per-expert form takes an XCD remap
   if (!g.valid) return;
   uint4 r1[RPT], r2[RPT], rgd[RPT];
   const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
-  constexpr bool LDNT = (BATCHED ? FQ_LDNT_SILU_BWD_B : FQ_LDNT_SILU_BWD) != 0;
-  constexpr int NT = BATCHED ? FQ_NT_SILU_BWD_B : FQ_NT_SILU_BWD;
+  constexpr bool LDNT = BATCHED ? Policy::kLoadHintSiluBwdBatched : Policy::kLoadHintSiluBwd;
+  constexpr int NT = BATCHED ? Policy::kStoreHintSiluBwdBatched : Policy::kStoreHintSiluBwd;
   const TilePart<RPT> tp = tile_part<RPT>(g);
   load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, N, tp.rows, r1, tp.sl.rgl);
   load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, N, tp.rows, r2, tp.sl.rgl);
@@ -280,8 +176,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   if (tp.sl.ws * (4 * RPT) < tp.rows) {  // waves beyond the last row of a partial tile keep zeros
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
-#if FQ_BWD_PIN
-      if constexpr (BATCHED || FQ_BWD_PIN > 1) {
+      if constexpr (BATCHED ? Policy::kPinBwdRowsBatched : Policy::kPinBwdRows) {
         // row s is widened after row s-1 is done (see fence_values): 136 -> 122 registers in the
         // per-expert form, which was capped at 128 and spilled 8 (16 KB of scratch traffic per tile,
         // a quarter of the output again in HBM writes: 97.1 -> 89.1 us at 65536 x 1024, 256 experts)
@@ -293,7 +188,6 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
           fence_packed(rgd[s]);
         }
       }
-#endif
       float a[8], b[8], go[8];
       unpack8(r1[s], a);
       unpack8(r2[s], b);
@@ -362,17 +256,17 @@ __global__ __launch_bounds__(256) void rowsum_kernel(const float* __restrict__ p
 //   y = (x * rstd[row]) * gamma[col]
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, int MODE, int NT>
-__global__ __launch_bounds__(2048 / FQ_RPT_RMS) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
+__global__ __launch_bounds__(2048 / Policy::kRowsPerThreadRmsnorm) void rmsnorm_quant_tile_kernel(const uint16_t* __restrict__ x,
                                                                  const uint16_t* __restrict__ gamma,
                                                                  const float* __restrict__ rstd, OutPtrs out,
                                                                  int64_t M, int n, int remap) {
-  constexpr int RPT = FQ_RPT_RMS;
+  constexpr int RPT = Policy::kRowsPerThreadRmsnorm;
   __shared__ TileShared<RPT> sh;
   BatchArgs none{nullptr, 0, 0};
   const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none, remap);
   if (!g.valid) return;
   uint4 raw[RPT];
-  load_rows<RPT, FQ_LDNT_RMSNORM != 0>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
+  load_rows<RPT, Policy::kLoadHintRmsnorm>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
   const int cg = threadIdx.x & 15;
   const int rg = threadIdx.x >> 4;
   float gm[8];
@@ -436,7 +330,7 @@ hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_b
   RowWeight w{weight, weight_bf16};
   const int64_t tiles = row_blocks * (n / kGroup);
   if (tiles == 0) return hipSuccess;
-  const dim3 grid((unsigned)tiles), block(2048 / FQ_RPT_FWD);
+  const dim3 grid((unsigned)tiles), block(2048 / Policy::kRowsPerThreadSiluFwd);
   const bool batched = counts != nullptr;
   const bool weighted = weight != nullptr;
   FQ_DISPATCH_KIND(kind, K,
@@ -482,7 +376,7 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
   const int64_t tiles = ((M + kGroup - 1) / kGroup) * (n / kGroup);
   if (tiles == 0) return hipSuccess;
-  const dim3 grid((unsigned)tiles), block(2048 / FQ_RPT_RMS);
+  const dim3 grid((unsigned)tiles), block(2048 / Policy::kRowsPerThreadRmsnorm);
   // transposed rows start every M bytes: off 16-byte boundaries their stores go out plain
   const bool aligned_rows = M % 16 == 0;
   // XCD remap (see resolve_tile): wide rows and several waves of workgroups
@@ -491,7 +385,7 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
         FQ_DISPATCH_BOOL(aligned_rows, A,
-          hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD, MD == 1 ? FQ_NT_RMSNORM_T : A ? FQ_NT_RMSNORM : (FQ_NT_RMSNORM & 2)>), grid,
+          hipLaunchKernelGGL((rmsnorm_quant_tile_kernel<K, R, MD, MD == 1 ? Policy::kStoreHintRmsnormCols : A ? Policy::kStoreHintRmsnorm : (Policy::kStoreHintRmsnorm & 2)>), grid,
                              block, 0, stream, (const uint16_t*)x, (const uint16_t*)gamma, rstd, out, M, n,
                              remap);))))
   return hipGetLastError();
