@@ -68,15 +68,9 @@ struct Policy {
   // ---- the per-expert SwiGLU backward widens row s of its packed inputs after row s-1 is done
   // (fence_values): 136 -> 122 registers, no spill under its cap of 128
   static constexpr bool kPinBwdRowsBatched = true;
-  static constexpr bool kPinBwdRows = false;
-
-  // ---- tile order across the XCDs (resolve_tile: 0 grid order, 1 one contiguous eighth of the
-  // tiles per XCD, 2 every eighth row block per XCD).  With partial tiles packed the per-expert
-  // SwiGLU backward runs 87.5 us in grid order, 89.3 with order 2 and 95.3 with order 1 (its
-  // launch is sized for one workgroup per 128 x 128 tile, so the workgroups that find no tile
-  // all land on the last XCDs); the forward is level.
-  static constexpr int kTileOrderSiluBwdBatched = 0;
-  static constexpr int kTileOrderSiluFwdBatched = 0;
+  static constexpr bool kPinBwdRows = true;
+  static constexpr bool kPinFwdRows = false;
+  static constexpr int kMinWavesSiluFwd = 1;  // waves per SIMD the forward SwiGLU kernel is compiled for
 
   // ---- row kernels: the outputs are written once (-3 to -7 % with the hint on the RMSNorm
   // backward, the bf16 SwiGLU rows and the 128x128 block quantiser); the loads of rows that a

@@ -395,21 +395,29 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
 }
 
 // NT: bit 0 = transposed codes, bit 1 = row-wise codes leave with the non-temporal hint
-template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0, bool LEAN = true, int NV = 1, bool TAIL_SYNC = false>
+// ALL_FULL: the launch has no partial tile (single matrix, M a multiple of 128): only the
+// mask-free path is compiled.  The ragged path costs registers the full one does not need
+// (SwiGLU forward: 77 against 62, i.e. three against four workgroups per CU).
+template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0, bool LEAN = true, int NV = 1, bool TAIL_SYNC = false,
+          bool ALL_FULL = false>
 __device__ __forceinline__ void quantize_tiles(const float (&v)[NV][RPT][8], const TileOut (&o)[NV],
                                                TileShared<RPT, NV>& sh) {
-  // workgroup-uniform choice of the mask-free path
-  const bool full = o[0].rows_valid == kGroup;
-  if (full) quantize_tiles_impl<KIND, ROUND, MODE, RPT, true, NT, LEAN, NV, TAIL_SYNC>(v, o, sh);
-  else quantize_tiles_impl<KIND, ROUND, MODE, RPT, false, NT, LEAN, NV, TAIL_SYNC>(v, o, sh);
+  if constexpr (ALL_FULL) {
+    quantize_tiles_impl<KIND, ROUND, MODE, RPT, true, NT, LEAN, NV, TAIL_SYNC>(v, o, sh);
+  } else {
+    // workgroup-uniform choice of the mask-free path
+    const bool full = o[0].rows_valid == kGroup;
+    if (full) quantize_tiles_impl<KIND, ROUND, MODE, RPT, true, NT, LEAN, NV, TAIL_SYNC>(v, o, sh);
+    else quantize_tiles_impl<KIND, ROUND, MODE, RPT, false, NT, LEAN, NV, TAIL_SYNC>(v, o, sh);
+  }
 }
 
 // one tile
-template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0, bool LEAN = true>
+template <int KIND, bool ROUND, int MODE, int RPT, int NT = 0, bool LEAN = true, bool ALL_FULL = false>
 __device__ __forceinline__ void quantize_tile(const float (&v)[RPT][8], const TileOut& o, TileShared<RPT>& sh) {
   const float (&vs)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(v);
   const TileOut (&os)[1] = reinterpret_cast<const TileOut (&)[1]>(o);
-  quantize_tiles<KIND, ROUND, MODE, RPT, NT, LEAN, 1, false>(vs, os, sh);
+  quantize_tiles<KIND, ROUND, MODE, RPT, NT, LEAN, 1, false, ALL_FULL>(vs, os, sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -449,6 +457,34 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
 // Column maxima stay per column, row maxima per row and column block: nothing else changes.
 __device__ __forceinline__ int pack_shift(int last_rows) { return last_rows <= 32 ? 2 : last_rows <= 64 ? 1 : 0; }
 
+// the 16-byte-chunk bookkeeping of an expert with `c` rows: padded rows, 128-row blocks, pack shift
+// of the last block and workgroups
+struct ExpertShape {
+  int pc, nb, shift, nw;
+};
+__device__ __forceinline__ ExpertShape expert_shape(int c, int ncb, int pad) {
+  ExpertShape e;
+  e.pc = (c + pad - 1) & -pad;  // pad is a power of two (1 or 16)
+  e.nb = (c + kGroup - 1) / kGroup;
+  e.shift = pack_shift(e.pc - (e.nb - 1) * kGroup);
+  e.nw = e.nb > 0 ? (e.nb - 1) * ncb + ((ncb + (1 << e.shift) - 1) >> e.shift) : 0;
+  return e;
+}
+
+constexpr int kLookupSteps = 16;  // 64 experts per step: the counts of up to 1024 experts are fetched together
+__device__ __forceinline__ void load_counts(const void* counts, int is_i64, int n_experts, int base0, int steps,
+                                            int (&cs)[kLookupSteps]) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int k = 0; k < kLookupSteps; ++k) {
+    cs[k] = 0;
+    if (k < steps) {
+      const int e = base0 + k * 64 + lane;
+      if (e < n_experts) cs[k] = load_count(counts, is_i64, e);
+    }
+  }
+}
+
 // Which tile does workgroup `wg` of a per-expert launch own?  Workgroups are numbered expert
 // after expert; an expert with nbk = ceil(count/128) row blocks takes (nbk - 1) * ncb workgroups
 // for its full row blocks (row block after row block, ncb column blocks each) and
@@ -456,15 +492,20 @@ __device__ __forceinline__ int pack_shift(int last_rows) { return last_rows <= 3
 // the device-side counts by a prefix scan that EVERY WAVE runs for itself, 64 experts per step
 // with the loads of up to sixteen steps in flight together: no LDS, no barrier, and every
 // thread of the workgroup ends with the same answer.  (A workgroup-wide scan with three
-// barriers cost 13 % of the batched SwiGLU forward.)  A workgroup beyond the last tile (the
-// launch is sized for one workgroup per 128 x 128 tile, packing needs fewer) or counts that
-// disagree with the host's yield expert = -1.
+// barriers cost 13 % of the batched SwiGLU forward, one wave scanning for the others 6 %.)
+// A workgroup beyond the last tile (the launch is sized for one workgroup per 128 x 128 tile,
+// packing needs fewer) or counts that disagree with the host's yield expert = -1.
+// Tiles are taken in grid order.  (Numbering them so that every XCD works on one contiguous
+// eighth of the real tiles - neighbouring row blocks of an expert share lines of the transposed
+// output, which one L2 merges and two do not: 11 % fewer bytes written by the per-expert SwiGLU
+// backward - needs the number of tiles first, one more pass over the counts, and measured
+// slower: 89.3 against 87.8 us for that kernel at 65536 x 1024 with 256 experts, 59 against
+// 51 us for gather+pad+quant.)
 // pad > 1: every expert's region starts at a multiple of pad rows (the reference's
 // permute-and-pad layout, pad = 16); 128 is a multiple of pad, so the number of
 // 128-row blocks of an expert does not change.
 __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int is_i64, int n_experts, int wg, int ncb,
                                                        int pad = 1) {
-  const int lane = threadIdx.x & 63;
   ExpertTile t;
   t.expert = -1;
   t.count = 0;
@@ -475,31 +516,17 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
   t.row_start = 0;
   t.tblock_start = 0;
   int run_rows = 0, run_blocks = 0, run_wgs = 0;
-  // the counts of up to 1024 experts (16 steps) are fetched together: one memory round
-  // trip however many steps the scan then takes
-  constexpr int kSteps = 16;
-  for (int base0 = 0; base0 < n_experts; base0 += 64 * kSteps) {
-    const int left = n_experts - base0;
-    const int steps = left >= 64 * kSteps ? kSteps : (left + 63) / 64;  // wave-uniform
-    int cs[kSteps];
-#pragma unroll
-    for (int k = 0; k < kSteps; ++k) {
-      cs[k] = 0;
-      if (k < steps) {
-        const int e = base0 + k * 64 + lane;
-        if (e < n_experts) cs[k] = load_count(counts, is_i64, e);
-      }
-    }
+  constexpr int kSteps = kLookupSteps;
+  int cs[kSteps];
+  // one chunk of up to 1024 experts whose counts sit in cs: true when the tile was found
+  auto scan_chunk = [&](int base0, int steps) -> bool {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
       if (k < steps) {
         const int base = base0 + k * 64;
         const int c = cs[k];
-        const int pc = (c + pad - 1) & -pad;  // pad is a power of two (1 or 16)
-        const int nb = (c + kGroup - 1) / kGroup;
-        const int shift = pack_shift(pc - (nb - 1) * kGroup);
-        const int kc = 1 << shift;
-        const int nw = nb > 0 ? (nb - 1) * ncb + ((ncb + kc - 1) >> shift) : 0;
+        const ExpertShape es = expert_shape(c, ncb, pad);
+        const int pc = es.pc, nb = es.nb, shift = es.shift, nw = es.nw;
         const int rows = wave_inclusive_scan(pc);
         const int blocks = wave_inclusive_scan(nb);
         const int wgs = wave_inclusive_scan(nw);
@@ -524,13 +551,20 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
             t.kc_shift = __builtin_amdgcn_readlane(shift, src);
             t.cb = (local - full) << t.kc_shift;
           }
-          return t;
+          return true;
         }
         run_rows += __builtin_amdgcn_readlane(rows, 63);
         run_blocks += __builtin_amdgcn_readlane(blocks, 63);
         run_wgs += __builtin_amdgcn_readlane(wgs, 63);
       }
     }
+    return false;
+  };
+  for (int base0 = 0; base0 < n_experts; base0 += 64 * kSteps) {
+    const int left = n_experts - base0;
+    const int steps = left >= 64 * kSteps ? kSteps : (left + 63) / 64;  // wave-uniform
+    load_counts(counts, is_i64, n_experts, base0, steps, cs);
+    if (scan_chunk(base0, steps)) return t;
   }
   return t;
 }

@@ -32,7 +32,7 @@ struct BatchArgs {
 // out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
 // backward's dx1|dx2)
 // remap: workgroup i runs on XCD i % 8; 1 = give every XCD one contiguous eighth of the
-// tiles instead of every eighth tile, 2 = give it every eighth row block (see below).  Which order of the tiles the memory system likes
+// tiles instead of every eighth tile (single-matrix kernels only).  Which order of the tiles the memory system likes
 // better depends on the kernel and the shape (measured: the RMSNorm tile kernel 4-18 %
 // faster with it at 16384 x 7168 and slower below ~2000 tiles or with narrow rows, the
 // per-expert SwiGLU backward 5 % faster; gather+pad+quant 18 % slower, the blockwise
@@ -49,17 +49,6 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
     // the first (G % 8, or 8) XCDs hold `per` tiles, the others one fewer
     const int full = (G & 7) ? (G & 7) : 8;
     id = xcd < full ? xcd * per + slot : full * per + (xcd - full) * (per - 1) + slot;
-  } else if (remap == 2) {
-    // runs of ncb consecutive tiles (one row block) stay on one XCD, the runs go round the XCDs:
-    // the neighbours in memory share an L2, and work that ends early in the numbering (a launch
-    // sized for more workgroups than there are tiles) is spread over all XCDs
-    const int G = (int)gridDim.x;
-    const int span = 8 * ncb;
-    if (id < G - G % span) {
-      const int xcd = id & 7, slot = id >> 3;
-      const int run = slot / ncb;
-      id = (run * 8 + xcd) * ncb + (slot - run * ncb);
-    }
   }
   g.kc_shift = 0;
   g.n_sub = 1;

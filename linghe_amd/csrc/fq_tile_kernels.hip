@@ -98,19 +98,21 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
 // ---------------------------------------------------------------------------
 // SwiGLU forward + quant.  y = (sigmoid(x1)*x1)*x2 [*w_row]   (fp32)
 // ---------------------------------------------------------------------------
-template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED>
-__global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
+// ALL_FULL: single matrix with M a multiple of 128 (see quantize_tiles)
+template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED, bool ALL_FULL>
+__global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd, Policy::kMinWavesSiluFwd) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {
   constexpr int RPT = Policy::kRowsPerThreadSiluFwd;
   __shared__ TileShared<RPT> sh;
-  const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch, BATCHED ? Policy::kTileOrderSiluFwdBatched : 0);
+  const TileGeom g = resolve_tile<BATCHED>(M, n / kGroup, n, batch);
   if (!g.valid) return;
   const int64_t ld = 2 * (int64_t)n;
   uint4 r1[RPT], r2[RPT];
   const uint16_t* p = x + g.row0 * ld + (int64_t)g.cb * kGroup;
   constexpr bool LDNT = BATCHED ? Policy::kLoadHintSiluFwdBatched : Policy::kLoadHintSiluFwd;
   constexpr int NT = MODE == 0 ? Policy::kStoreHintSiluFwdRows : MODE == 1 ? Policy::kStoreHintSiluFwdCols : BATCHED ? Policy::kStoreHintSiluFwdBatched : Policy::kStoreHintSiluFwd;
-  const TilePart<RPT> tp = tile_part<RPT>(g);
+  TilePart<RPT> tp = tile_part<RPT>(g);
+  if constexpr (ALL_FULL) tp.rows = kGroup;  // a constant: the masked loads and the zero fill fold away
   load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, ld, tp.rows, r1, tp.sl.rgl);
   load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, ld, tp.rows, r2, tp.sl.rgl);
   const int rg = tp.sl.rgl;
@@ -122,6 +124,13 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd) void silu_qua
   if (tp.sl.ws * (4 * RPT) < tp.rows) {  // waves beyond the last row of a partial tile keep zeros
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
+      if constexpr (Policy::kPinFwdRows) {
+        if (s > 0) {  // row s is widened after row s-1 is done (see fence_values)
+          fence_values(v[s - 1]);
+          fence_packed(r1[s]);
+          fence_packed(r2[s]);
+        }
+      }
       float a[8], b[8];
       unpack8(r1[s], a);
       unpack8(r2[s], b);
@@ -138,7 +147,7 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd) void silu_qua
       }
     }
   }
-  quantize_tile<KIND, ROUND, MODE, RPT, NT>(v, make_out(out, g, n, g.cb), sh);
+  quantize_tile<KIND, ROUND, MODE, RPT, NT, true, ALL_FULL>(v, make_out(out, g, n, g.cb), sh);
 }
 
 // ---------------------------------------------------------------------------
@@ -155,13 +164,14 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   constexpr int RPT = 4;
   const int nb = n / kGroup;
   const int64_t N = 2 * (int64_t)n;
-  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch, BATCHED ? Policy::kTileOrderSiluBwdBatched : 0);  // the per-expert form takes an XCD remap
+  const TileGeom g = resolve_tile<BATCHED>(M, nb, N, batch);
   if (!g.valid) return;
   uint4 r1[RPT], r2[RPT], rgd[RPT];
   const uint16_t* p = x + g.row0 * N + (int64_t)g.cb * kGroup;
   constexpr bool LDNT = BATCHED ? Policy::kLoadHintSiluBwdBatched : Policy::kLoadHintSiluBwd;
   constexpr int NT = BATCHED ? Policy::kStoreHintSiluBwdBatched : Policy::kStoreHintSiluBwd;
-  const TilePart<RPT> tp = tile_part<RPT>(g);
+  TilePart<RPT> tp = tile_part<RPT>(g);
+  if constexpr (!BATCHED) tp.rows = kGroup;  // single matrix: M % 128 == 0
   load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, N, tp.rows, r1, tp.sl.rgl);
   load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, N, tp.rows, r2, tp.sl.rgl);
   load_rows<RPT, LDNT>(gr + g.row0 * n + (int64_t)tp.cb * kGroup, n, tp.rows, rgd, tp.sl.rgl);
@@ -228,7 +238,8 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
     // with it, so it quantises one tile after the other.
     __shared__ TileShared<RPT, 2> sh;
     const TileOut outs[2] = {make_out(out, g, N, g.cb), make_out(out, g, N, nb + g.cb)};
-    quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 2>(d, outs, sh);
+    // the single-matrix form takes M % 128 == 0 only (as the reference): no partial tile
+    quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 2, false, true>(d, outs, sh);
   } else {
     __shared__ TileShared<RPT> sh;
     const TileOut o1[1] = {make_out(out, g, N, g.cb)};
@@ -333,13 +344,15 @@ hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_b
   const dim3 grid((unsigned)tiles), block(2048 / Policy::kRowsPerThreadSiluFwd);
   const bool batched = counts != nullptr;
   const bool weighted = weight != nullptr;
+  const bool all_full = !batched && M % kGroup == 0;
   FQ_DISPATCH_KIND(kind, K,
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
         FQ_DISPATCH_BOOL(batched, B,
           FQ_DISPATCH_BOOL(weighted, W,
-            hipLaunchKernelGGL((silu_quant_fwd_kernel<K, R, MD, B, W>), grid, block, 0, stream,
-                               (const uint16_t*)x, w, out, M, n, b);)))))
+            FQ_DISPATCH_BOOL(all_full, AF,
+              hipLaunchKernelGGL((silu_quant_fwd_kernel<K, R, MD, B, W, AF && !B>), grid, block, 0, stream,
+                                 (const uint16_t*)x, w, out, M, n, b);))))))
   return hipGetLastError();
 }
 
