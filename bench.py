@@ -129,6 +129,7 @@ def build_cases(names, dev):
     add("cfg1_pow2", build=lambda: rms_quant_case("cfg1_pow2", configs.cfg1_rmsnorm_quant(), 2, True))
     add("cfg5b", build=lambda: rms_quant_case("cfg5b", cfg5(), 2))
     add("cfg5c", build=lambda: rms_quant_case("cfg5c", cfg5(), 1))
+    add("cfg5b_pow2", build=lambda: rms_quant_case("cfg5b_pow2", cfg5(), 2, True))
     # output_mode 0 (row-wise codes only: the first forward of a layer that will be recomputed)
     add("cfg1_mode0", build=lambda: rms_quant_case("cfg1_mode0", configs.cfg1_rmsnorm_quant(), 0))
     add("cfg5_mode0", build=lambda: rms_quant_case("cfg5_mode0", cfg5(), 0))
@@ -735,7 +736,7 @@ def load_traffic_table():
 
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
-       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
+       "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg5b_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed",
        "stream_read", "stream_copy"]
 
