@@ -23,7 +23,8 @@ Prints ONE short JSON line on stdout (under 4000 characters): the headline
 metric is us/call of RMSNorm + 1x128 quant forward on bf16 [8192, 2048]
 (output_mode 2) with its roofline and CPU baseline; the other configurations
 appear as name -> [us, fraction of peak, fraction of the no-work kernel's rate].
-Every field of every configuration goes to gpurun_out/bench_full.json; stderr
+Every field of every configuration goes to bench_full.json in the results folder
+(RESULTS_DIR); stderr
 carries one summary line per configuration.
 """
 from __future__ import annotations
@@ -455,8 +456,8 @@ def build_cases(names, dev):
         add(_n, build=lambda _n=_n: plain_quant_case(_n))
 
     # ---------------------------------------------------------------- next row: RMSNorm + router GEMM + quant
-    def router_case(packed=False):
-        M, N, K = 8192, 256, 2048
+    def router_case(packed=False, shape=(8192, 256, 2048), name=None):
+        M, N, K = shape
         g = torch.Generator().manual_seed(1104)
         x_cpu = (torch.randn(M, K, generator=g) ** 2).to(torch.bfloat16)
         nw_cpu = torch.randn(K, generator=g).to(torch.bfloat16)
@@ -486,7 +487,7 @@ def build_cases(names, dev):
             from oracle import fq_oracle as O
             return O.rms_gemm_block_quant_forward(x_cpu, nw_cpu, rw_cpu)
 
-        c = Case("next_router_packed" if packed else "next_router",
+        c = Case(name or ("next_router_packed" if packed else "next_router"),
                  "triton_rms_norm_fp32_gemm_block_quant_forward(output_mode=0%s)"
                  % (", packed_route_weight=..." if packed else ""), [M, N, K],
                  configs.rw_router(M, N, K), make_set, launch, cpu_fn)
@@ -495,6 +496,8 @@ def build_cases(names, dev):
 
     add("next_router", build=router_case)
     add("next_router_packed", build=lambda: router_case(True))
+    # a wide router: more than 512 logits run as one launch per 512 (virtual) columns, x re-read by each
+    add("next_router_wide", build=lambda: router_case(False, (2048, 2048, 2048), "next_router_wide"))
 
     # ---------------------------------------------------------------- the no-work stream kernel on a known size
     # (the read / copy rates of the memory system, and the calibration of FETCH_SIZE / WRITE_SIZE)
@@ -737,7 +740,7 @@ def load_traffic_table():
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
        "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg5b_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
-       "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed",
+       "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed", "next_router_wide",
        "stream_read", "stream_copy"]
 
 
@@ -859,14 +862,15 @@ def encode_line(line):
     return text
 
 
+RESULTS_DIR = "gpurun_out"  # folder, beside this file, that side results are written to
 MAX_LINE_CHARS = 4000  # the last stdout line must fit the window a harness keeps of stdout
 HEADLINE_CONFIGS = ("cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg5a", "cfg5b", "cfg5c")
 
 
 def write_full_results(results, args):
-    """Every field of every configuration: to gpurun_out/bench_full.json, or, when that cannot be
-    written, as one JSON object per configuration on stderr.  The stdout line stays short."""
-    out_dir = os.path.join(ROOT, "gpurun_out")
+    """Every field of every configuration: to bench_full.json in the results folder, or, when that
+    cannot be written, as one JSON object per configuration on stderr.  The stdout line stays short."""
+    out_dir = os.path.join(ROOT, RESULTS_DIR)
     try:
         os.makedirs(out_dir, exist_ok=True)
         with open(os.path.join(out_dir, "bench_full.json"), "w") as f:
@@ -921,7 +925,7 @@ def headline_line(results, steps, warmup, settle_us):
                        for name, r in results.items()}
     line["from_idle_us"] = {name: r["us_per_call_from_idle"] for name, r in results.items()
                             if "us_per_call_from_idle" in r}
-    line["full_results"] = "gpurun_out/bench_full.json"
+    line["full_results"] = RESULTS_DIR + "/bench_full.json"
     return line
 
 
