@@ -78,6 +78,16 @@ def test_c_side_validation_without_gpu():
     # hidden size too large for the row kernels
     rc = L.fq_rmsnorm_fwd(None, None, None, None, 4, 16384, 1e-6, 0, None)
     assert rc == -2
+    # router weight packing: K not a multiple of 128, N beyond the limit, NULL buffers
+    assert L.fq_pack_router_weight(None, 0, None, 100, 128, None) == -2
+    assert L.fq_pack_router_weight(None, 0, None, 2048, 8192 + 128, None) == -2
+    assert L.fq_pack_router_weight(None, 0, None, 2048, 256, None) == -1
+    assert L.fq_rmsnorm_router_quant_fwd_packed(None, None, None, 0, None, None, None, None, None, 128, 2048, 100,
+                                                1e-6, 0, 0, None) == -2
+    # the no-work kernel's variants: chunks per lane 4 / 8 / 16 only, order 0..2
+    assert L.fq_stream_rw_variant(None, 0, None, 0, None, 4, 0, 0, 0, 0, None) == -1          # no sink
+    assert L.fq_stream_rw_variant(None, 16, None, 0, None, 5, 0, 0, 0, 0, None) == -1
+    assert L.fq_stream_rw_variant(None, 24, None, 0, None, 4, 0, 0, 0, 0, None) == -2         # not a multiple of 16
     # 128x128 block quant needs whole blocks of rows
     rc = L.fq_block_quant(None, None, None, 100, 256, 0, 0, None)
     assert rc == -2 and b"128" in L.fq_last_error()
