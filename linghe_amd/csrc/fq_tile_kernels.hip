@@ -116,12 +116,12 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd, Policy::kMinW
   load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, ld, tp.rows, r1, tp.sl.rgl);
   load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, ld, tp.rows, r2, tp.sl.rgl);
   const int rg = tp.sl.rgl;
+  // Every wave does the arithmetic, also one whose rows all lie beyond the last row of a partial tile
+  // (its inputs read as zeros and give zeros): a branch around the arithmetic keeps the zero-filled results
+  // and the packed inputs alive side by side and costs 13-20 registers (73 -> 60 in the per-expert form:
+  // three -> four workgroups per CU), while skipping the arithmetic gained nothing measurable.
   float v[RPT][8];
-#pragma unroll
-  for (int s = 0; s < RPT; ++s)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[s][j] = 0.f;
-  if (tp.sl.ws * (4 * RPT) < tp.rows) {  // waves beyond the last row of a partial tile keep zeros
+  {
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
       if constexpr (Policy::kPinFwdRows) {
@@ -179,11 +179,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   const int rg = tp.sl.rgl;
   float d[2][RPT][8];  // dx1, dx2
   float my_dw = 0.f;
-#pragma unroll
-  for (int s = 0; s < RPT; ++s)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) d[0][s][j] = d[1][s][j] = 0.f;
-  if (tp.sl.ws * (4 * RPT) < tp.rows) {  // waves beyond the last row of a partial tile keep zeros
+  {  // every wave does the arithmetic (see the forward kernel): zero inputs give zero results
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
       if constexpr (BATCHED ? Policy::kPinBwdRowsBatched : Policy::kPinBwdRows) {
