@@ -63,14 +63,18 @@ struct Policy {
   // 16384 x 7168 (110.5 us either way, 58.9 / 58.5 us with the statistic given) and 2 % behind at
   // 8192 x 2048 (18.3 / 18.0 us), so it runs with 4.
   static constexpr int kRowsPerThreadSiluFwd = 4;
+  // Rows of a 128x128 tile per thread in the plain blockwise quantiser: 8 (256 threads) for the
+  // dense form (4 rows: 13.2 -> 13.9 us on 8192x4096), 4 (512 threads) for the per-expert form,
+  // which waits on its lookup and gains from more waves per CU (31.3 -> 30.9 us, 32 experts).
+  static constexpr int kRowsPerThreadBlockwise = 8;
+  static constexpr int kRowsPerThreadBlockwiseBatched = 4;
   static constexpr int kRowsPerThreadRmsnorm = 4;
 
-  // ---- the per-expert SwiGLU backward widens row s of its packed inputs after row s-1 is done
-  // (fence_values): 136 -> 122 registers, no spill under its cap of 128
+  // ---- the SwiGLU backwards widen row s of their packed inputs after row s-1 is done (fence_values):
+  // without it the per-expert form needed 136 registers under its cap of 128 and spilled; with it (and no
+  // branch around the arithmetic) 105, the single-matrix form 100
   static constexpr bool kPinBwdRowsBatched = true;
   static constexpr bool kPinBwdRows = true;
-  static constexpr bool kPinFwdRows = false;
-  static constexpr int kMinWavesSiluFwd = 1;  // waves per SIMD the forward SwiGLU kernel is compiled for
 
   // ---- row kernels: the outputs are written once (-3 to -7 % with the hint on the RMSNorm
   // backward, the bf16 SwiGLU rows and the 128x128 block quantiser); the loads of rows that a

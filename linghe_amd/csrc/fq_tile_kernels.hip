@@ -15,9 +15,9 @@ namespace fq {
 // plain blockwise quant
 // ---------------------------------------------------------------------------
 template <int KIND, bool ROUND, int MODE, bool BATCHED>
-__global__ __launch_bounds__(256) void blockwise_quant_kernel(const uint16_t* __restrict__ x, OutPtrs out,
-                                                              int64_t M, int N, BatchArgs batch) {
-  constexpr int RPT = 8;
+__global__ __launch_bounds__(2048 / (BATCHED ? Policy::kRowsPerThreadBlockwiseBatched : Policy::kRowsPerThreadBlockwise))
+void blockwise_quant_kernel(const uint16_t* __restrict__ x, OutPtrs out, int64_t M, int N, BatchArgs batch) {
+  constexpr int RPT = BATCHED ? Policy::kRowsPerThreadBlockwiseBatched : Policy::kRowsPerThreadBlockwise;
   __shared__ TileShared<RPT> sh;
   const TileGeom g = resolve_tile<BATCHED>(M, N / kGroup, N, batch);
   if (!g.valid) return;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
 // ---------------------------------------------------------------------------
 // ALL_FULL: single matrix with M a multiple of 128 (see quantize_tiles)
 template <int KIND, bool ROUND, int MODE, bool BATCHED, bool WEIGHTED, bool ALL_FULL>
-__global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd, Policy::kMinWavesSiluFwd) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
+__global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd) void silu_quant_fwd_kernel(const uint16_t* __restrict__ x, RowWeight weight,
                                                              OutPtrs out, int64_t M, int n, BatchArgs batch) {
   constexpr int RPT = Policy::kRowsPerThreadSiluFwd;
   __shared__ TileShared<RPT> sh;
@@ -124,13 +124,6 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd, Policy::kMinW
   {
 #pragma unroll
     for (int s = 0; s < RPT; ++s) {
-      if constexpr (Policy::kPinFwdRows) {
-        if (s > 0) {  // row s is widened after row s-1 is done (see fence_values)
-          fence_values(v[s - 1]);
-          fence_packed(r1[s]);
-          fence_packed(r2[s]);
-        }
-      }
       float a[8], b[8];
       unpack8(r1[s], a);
       unpack8(r2[s], b);
@@ -301,8 +294,9 @@ hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, fl
   BatchArgs b{counts, counts_i64, n_experts};
   const int64_t tiles = row_blocks * (N / kGroup);
   if (tiles == 0) return hipSuccess;
-  const dim3 grid((unsigned)tiles), block(256);
   const bool batched = counts != nullptr;
+  const dim3 grid((unsigned)tiles),
+      block(2048 / (batched ? Policy::kRowsPerThreadBlockwiseBatched : Policy::kRowsPerThreadBlockwise));
   FQ_DISPATCH_KIND(kind, K,
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
