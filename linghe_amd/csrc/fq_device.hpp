@@ -7,6 +7,30 @@
 
 namespace fq {
 
+// Work-item and workgroup numbers straight from the hardware registers and the kernel's hidden
+// arguments.  HIP's threadIdx / blockIdx / gridDim go through device-library functions, and this
+// build cannot inline those (the library is compiled with the packed-fp32 feature that the build
+// switches off, and a function is not inlined into a caller that lacks one of its target
+// features): every use was a real call, with the calling convention's constraints on the
+// registers live around it.
+__device__ __forceinline__ unsigned tid_x() { return __builtin_amdgcn_workitem_id_x(); }
+__device__ __forceinline__ unsigned wg_x() { return __builtin_amdgcn_workgroup_id_x(); }
+// The same, opaque to the compiler, for the 128x128 tile code.  From the plain form the compiler
+// derives every lane offset and mask of a tile kernel early and keeps them alive (and moves them
+// out of any loop over tiles, some thirty registers); with this one each use site starts from
+// its own copy of the register and the derived values die where they are used: 4-9 registers
+// fewer in every tile kernel (SwiGLU forward 56-61 -> 51-56, RMSNorm tile kernel 58-62 -> 52),
+// 1-5 % less time in the SwiGLU and RMSNorm tile kernels.
+__device__ __forceinline__ unsigned tile_tid() {
+  unsigned t = tid_x();
+  asm volatile("" : "+v"(t));
+  return t;
+}
+// number of workgroups of the launch: the first hidden kernel argument (code object v5 and later)
+__device__ __forceinline__ unsigned n_wg_x() {
+  return ((const __attribute__((address_space(4))) uint32_t*)__builtin_amdgcn_implicitarg_ptr())[0];
+}
+
 constexpr int kGroup = 128;           // 1x128 / 128x1 quantisation group
 constexpr float kScaleFloor = 1e-30f;  // linghe/tools/util.py:58-60
 

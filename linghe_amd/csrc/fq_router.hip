@@ -57,7 +57,7 @@ struct RouterShared {
 // flight together), the arithmetic of the row kernels: 8-element group sums added
 // in double, so the value does not depend on the split
 __device__ __forceinline__ void router_rows_rstd(const uint16_t* rows, int n, float eps, float (&out)[4]) {
-  const int lane = threadIdx.x & 63;
+  const int lane = tid_x() & 63;
   const int chunks = n >> 3;
   double ss[4] = {0.0, 0.0, 0.0, 0.0};
   for (int c0 = 0; c0 < chunks; c0 += 256) {
@@ -89,7 +89,7 @@ template <bool FP32W>
 __global__ __launch_bounds__(256) void pack_router_weight_kernel(const void* __restrict__ wr,
                                                                  uint4* __restrict__ packed, int K, int vcol0,
                                                                  int vtiles) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // piece number inside the chunk
+  const int64_t idx = (int64_t)wg_x() * 256 + tid_x();  // piece number inside the chunk
   const int64_t total = (int64_t)vtiles * 32 * K / 8;
   if (idx >= total) return;
   const int lane = (int)(idx & 63);
@@ -146,9 +146,9 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
     uint16_t* __restrict__ y, float* __restrict__ rstd_out, LogitsOut lout, uint8_t* __restrict__ q,
     float* __restrict__ s, int64_t M, int K, float eps) {
   __shared__ RouterShared sh;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int64_t row0 = (int64_t)blockIdx.x * kRouterRows;
+  const int lane = tid_x() & 63;
+  const int wave = tid_x() >> 6;
+  const int64_t row0 = (int64_t)wg_x() * kRouterRows;
 
   constexpr int NT = TPW;
   constexpr int RPT = 8 / WAVES;  // rows per thread: 2 with 4 waves, 1 with 8
@@ -168,8 +168,8 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_kernel(
 
   // producer side: thread (rg, cg) holds rows RPT rg .. and columns 8 cg .. 8 cg + 7 of
   // the k block, so 16 lanes read, and write, 256 (128 for the codes) contiguous bytes
-  const int cg = threadIdx.x & 15;
-  const int rg = threadIdx.x >> 4;
+  const int cg = tid_x() & 15;
+  const int rg = tid_x() >> 4;
   const float r0 = sh.rstd[RPT * rg], r1 = sh.rstd[RPT * rg + RPT - 1];
   const uint16_t* xrow = x + (row0 + RPT * rg) * K + cg * 8;
   uint16_t* yrow = y + (row0 + RPT * rg) * K + cg * 8;
@@ -309,15 +309,15 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
     float* __restrict__ s, int64_t M, int K, float eps) {
   __shared__ RouterShared sh;
   __shared__ uint4 sgamma[KB * 16];  // gamma, 8 columns per piece
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int64_t row0 = (int64_t)blockIdx.x * kRouterRows;
+  const int lane = tid_x() & 63;
+  const int wave = tid_x() >> 6;
+  const int64_t row0 = (int64_t)wg_x() * kRouterRows;
   constexpr int NT = TPW;
   constexpr int RPT = 8 / WAVES;
   constexpr int kAhead = 6;  // k blocks of x in flight ahead of the one worked on
   constexpr int kWAhead = WDEPTH - 1;  // k blocks of W in flight ahead of the one worked on
-  const int cg = threadIdx.x & 15;
-  const int rg = threadIdx.x >> 4;
+  const int cg = tid_x() & 15;
+  const int rg = tid_x() >> 4;
   const uint16_t* xrow = x + (row0 + RPT * rg) * K + cg * 8;
   const int aj = cg & 7;
   const int ahalf = cg >> 3;
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(64 * WAVES) void rmsnorm_router_quant_resident_kern
 #pragma unroll
   for (int d = 0; d < kAhead; ++d)
     if (d < kblocks) fetch_x(d, xr[d]);
-  for (int p = threadIdx.x; p < kblocks * 16; p += 64 * WAVES) sgamma[p] = *(const uint4*)(gamma + p * 8);
+  for (int p = tid_x(); p < kblocks * 16; p += 64 * WAVES) sgamma[p] = *(const uint4*)(gamma + p * 8);
   __syncthreads();
 
   // ---- sweep 1, software pipelined: the A operands of block kb + 1 are produced

@@ -37,8 +37,8 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, RowShared<T>& sh,
   a = wave_sum(a);
   b = wave_sum(b);
   if constexpr (T > 64) {
-    const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) {
+    const int wave = tid_x() >> 6;
+    if ((tid_x() & 63) == 0) {
       sh.red[parity][0][wave] = a;
       sh.red[parity][1][wave] = b;
     }
@@ -59,8 +59,8 @@ __device__ __forceinline__ void block_sum2(double& a, float& b, RowShared<T>& sh
   a = wave_sum_d(a);
   b = wave_sum(b);
   if constexpr (T > 64) {
-    const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) {
+    const int wave = tid_x() >> 6;
+    if ((tid_x() & 63) == 0) {
       sh.redd[parity][wave] = a;
       sh.red[parity][1][wave] = b;
     }
@@ -79,7 +79,7 @@ template <int T, int NCHUNK, bool STREAM = false>
 __device__ __forceinline__ void load_row(const uint16_t* row, int n, uint4 (&raw)[NCHUNK]) {
 #pragma unroll
   for (int k = 0; k < NCHUNK; ++k) {
-    const int c = threadIdx.x + k * T;
+    const int c = tid_x() + k * T;
     raw[k] = make_uint4(0, 0, 0, 0);
     if (c * 8 < n) raw[k] = load16<STREAM>(row + c * 8);
   }
@@ -95,7 +95,7 @@ __device__ __forceinline__ void load_row_clamped(const uint16_t* row, int n, uin
   const int last = (n >> 3) - 1;
 #pragma unroll
   for (int k = 0; k < NCHUNK; ++k) {
-    const int c = threadIdx.x + k * T;
+    const int c = tid_x() + k * T;
     raw[k] = load16<STREAM>(row + (c < last ? c : last) * 8);
   }
 }
@@ -136,7 +136,7 @@ __device__ __forceinline__ double sumsq_live(const uint4 (&raw)[NCHUNK], int n) 
 #pragma unroll
   for (int k = 0; k < NCHUNK; ++k) {
     const float part = sumsq8(raw[k]);
-    ss += (double)((((int)threadIdx.x & (T - 1)) + k * T) * 8 < n ? part : 0.f);  // T a power of two; a wave-per-row kernel passes T = 64
+    ss += (double)((((int)tid_x() & (T - 1)) + k * T) * 8 < n ? part : 0.f);  // T a power of two; a wave-per-row kernel passes T = 64
   }
   return ss;
 }
@@ -150,17 +150,17 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
                                                         float* __restrict__ scale, float* __restrict__ rstd,
                                                         int64_t M, int n, float eps, int rows_per_wg) {
   __shared__ RowShared<T> sh;
-  const int tid = threadIdx.x;
+  const int tid = tid_x();
   uint4 gm[NCHUNK];
   load_row<T, NCHUNK>(gamma, n, gm);
-  const int64_t G = gridDim.x;  // rows b, b + G, b + 2G, ... with b the workgroup's logical index:
+  const int64_t G = n_wg_x();  // rows b, b + G, b + 2G, ... with b the workgroup's logical index:
   // workgroup i runs on XCD i % 8, and every XCD takes one contiguous eighth of the
   // indices in the quantising form (3-7 % faster; the bf16 form is 8-20 % slower with it)
-  int64_t r0 = blockIdx.x;
+  int64_t r0 = wg_x();
   if constexpr (OUT == 1 && Policy::kXcdContiguousRowQuant) {
-    const int Gi = (int)gridDim.x;
+    const int Gi = (int)n_wg_x();
     const int per = (Gi + 7) >> 3;
-    const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
+    const int xcd = (int)wg_x() & 7, slot = (int)wg_x() >> 3;
     const int full = (Gi & 7) ? (Gi & 7) : 8;
     r0 = xcd < full ? xcd * per + slot : full * per + (xcd - full) * (per - 1) + slot;
   }
@@ -242,13 +242,13 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
 template <int U>
 __global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict__ x, float* __restrict__ rstd,
                                                      int64_t M, int n, float eps) {
-  const int lane = threadIdx.x;
+  const int lane = tid_x();
   const int chunks = n >> 3;
   // Rows are taken from the END of the matrix backwards.  The tile kernel that follows
   // walks the matrix forwards, so it starts with the rows this kernel read last, which
   // are the ones still in the last-level cache: for an input about the size of that
   // cache roughly half of the second read never reaches HBM.
-  for (int64_t k = blockIdx.x; k < M; k += gridDim.x) {
+  for (int64_t k = wg_x(); k < M; k += n_wg_x()) {
     const int64_t row = M - 1 - k;
     const uint4* p = (const uint4*)(x + row * n);
     double ss = 0.0;
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
                                                         uint16_t* __restrict__ dx, float* __restrict__ dg_part,
                                                         int64_t M, int n, float eps, int rows_per_wg) {
   __shared__ RowShared<T> sh;
-  const int tid = threadIdx.x;
+  const int tid = tid_x();
   const int chunks = n >> 3;
   // A thread's chunk k is column chunk tid + k*T.  Beyond the end of the row it reads the
   // row's last chunk again (a valid address, no branch) and takes part with gamma = 0:
@@ -306,9 +306,9 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[k][j] = 0.f;
 
-  // rows blockIdx.x, blockIdx.x + G, blockIdx.x + 2G, ...: at any moment the
+  // rows wg_x(), wg_x() + G, wg_x() + 2G, ...: at any moment the
   // workgroups of the grid work on neighbouring rows (one moving front in memory)
-  const int64_t G = gridDim.x;
+  const int64_t G = n_wg_x();
   (void)rows_per_wg;
 
   // One row in registers at a time (about 100 of them with two chunks per thread), so
@@ -316,7 +316,7 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
   // the next row's packed data into a second register set spills (142 -> 198 us at
   // 16384 x 7168 with 512 threads, 155 -> 179 us with 256 threads and four chunks).
   int parity = 0;
-  for (int64_t row = blockIdx.x; row < M; row += G) {
+  for (int64_t row = wg_x(); row < M; row += G) {
     uint4 rx[NCHUNK], rg[NCHUNK];
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
   for (int k = 0; k < NCHUNK; ++k) {
     const int c = tid + k * T;
     if (c * 8 < n) {
-      float4* dst = (float4*)(dg_part + (int64_t)blockIdx.x * n + c * 8);
+      float4* dst = (float4*)(dg_part + (int64_t)wg_x() * n + c * 8);
       dst[0] = make_float4(acc[k][0], acc[k][1], acc[k][2], acc[k][3]);
       dst[1] = make_float4(acc[k][4], acc[k][5], acc[k][6], acc[k][7]);
     }
@@ -389,8 +389,8 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_wave_kernel(const uint16_t* _
                                                                float* __restrict__ dg_part, int64_t M, int n,
                                                                float eps) {
   __shared__ float4 combine[3][NCHUNK * 2][64];  // waves 1..3: [chunk half][lane]
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int lane = tid_x() & 63;
+  const int wave = tid_x() >> 6;
   const int chunks = n >> 3;
   float w[NCHUNK][8];  // gamma, unpacked once; zero beyond the end of the row
 #pragma unroll
@@ -406,8 +406,8 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_wave_kernel(const uint16_t* _
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[k][j] = 0.f;
 
-  const int64_t stride = (int64_t)gridDim.x * 4;
-  for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < M; row += stride) {
+  const int64_t stride = (int64_t)n_wg_x() * 4;
+  for (int64_t row = (int64_t)wg_x() * 4 + wave; row < M; row += stride) {
     uint4 rx[NCHUNK], rg[NCHUNK];
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_wave_kernel(const uint16_t* _
       }
       const int c = lane + k * 64;
       if (c < chunks) {
-        float4* dst = (float4*)(dg_part + (int64_t)blockIdx.x * n + c * 8);
+        float4* dst = (float4*)(dg_part + (int64_t)wg_x() * n + c * 8);
         dst[0] = make_float4(acc[k][0], acc[k][1], acc[k][2], acc[k][3]);
         dst[1] = make_float4(acc[k][4], acc[k][5], acc[k][6], acc[k][7]);
       }
@@ -484,9 +484,9 @@ constexpr int kColsumSlices = 16;
 __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ part, float* __restrict__ out,
                                                       int P, int n) {
   __shared__ float red[kColsumSlices][64];
-  const int lane = threadIdx.x & 63;
-  const int col = blockIdx.x * 64 + lane;
-  const int slice = threadIdx.x >> 6;
+  const int lane = tid_x() & 63;
+  const int col = wg_x() * 64 + lane;
+  const int slice = tid_x() >> 6;
   float acc = 0.f;
   if (col < n) {
     const float* src = part + col;
@@ -516,9 +516,9 @@ __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ 
 template <int KIND, bool ROUND>
 __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
                                                           float* __restrict__ s, int64_t n_groups) {
-  const int64_t g0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
-  const int64_t stride = ((int64_t)gridDim.x * 256) >> 4;
-  const int sub = threadIdx.x & 15;
+  const int64_t g0 = ((int64_t)wg_x() * 256 + tid_x()) >> 4;
+  const int64_t stride = ((int64_t)n_wg_x() * 256) >> 4;
+  const int sub = tid_x() & 15;
   const int64_t limit = (n_groups + stride - 1) / stride * stride;  // keep the 16 lanes of a row together
   for (int64_t g = g0; g < limit; g += stride) {
     const bool ok = g < n_groups;
@@ -744,9 +744,9 @@ hipError_t launch_group_quant(const void* x, void* q, float* s, int64_t n_groups
 template <bool WEIGHTED>
 __global__ __launch_bounds__(64) void swiglu_fwd_rows_kernel(const uint16_t* __restrict__ x, RowWeight weight,
                                                              uint16_t* __restrict__ out, int64_t M, int n) {
-  const int lane = threadIdx.x;
+  const int lane = tid_x();
   const int chunks = n >> 3;
-  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+  for (int64_t row = wg_x(); row < M; row += n_wg_x()) {
     const uint16_t* p = x + row * 2 * (int64_t)n;
     float w = 1.0f;
     if constexpr (WEIGHTED) w = load_weight(weight, row);
@@ -782,9 +782,9 @@ __global__ __launch_bounds__(64) void swiglu_bwd_rows_kernel(const uint16_t* __r
                                                              const uint16_t* __restrict__ x, RowWeight weight,
                                                              uint16_t* __restrict__ dx, void* __restrict__ dw,
                                                              int64_t M, int n) {
-  const int lane = threadIdx.x;
+  const int lane = tid_x();
   const int chunks = n >> 3;
-  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+  for (int64_t row = wg_x(); row < M; row += n_wg_x()) {
     const uint16_t* p = x + row * 2 * (int64_t)n;
     const uint16_t* gp = gr + row * (int64_t)n;
     uint16_t* o = dx + row * 2 * (int64_t)n;
@@ -875,8 +875,8 @@ __global__ __launch_bounds__(256) void block_quant_kernel(const uint16_t* __rest
                                                           float* __restrict__ s, int N) {
   __shared__ float wmax[4];
   const int ncb = N / kGroup;
-  const int rb = blockIdx.x / ncb, cb = blockIdx.x - rb * ncb;
-  const int cg = threadIdx.x & 15, rg = threadIdx.x >> 4;
+  const int rb = wg_x() / ncb, cb = wg_x() - rb * ncb;
+  const int cg = tid_x() & 15, rg = tid_x() >> 4;
   const uint8_t* src = (const uint8_t*)(x + ((int64_t)rb * kGroup) * N + (int64_t)cb * kGroup);
   uint8_t* dst = q + ((int64_t)rb * kGroup) * N + (int64_t)cb * kGroup;
   const uint32_t off = (uint32_t)(rg * 8) * (uint32_t)N + (uint32_t)cg * 8u;  // in elements
@@ -892,12 +892,12 @@ __global__ __launch_bounds__(256) void block_quant_kernel(const uint16_t* __rest
     for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(a[j]));
   }
   m = wave_max(m);
-  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
+  if ((tid_x() & 63) == 0) wmax[tid_x() >> 6] = m;
   __syncthreads();
   m = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
   const float sc = make_scale<KIND, ROUND>(m);
   const Quantum<ROUND> d = make_quantum<ROUND>(sc);
-  if (threadIdx.x == 0) s[(int64_t)rb * ncb + cb] = sc;
+  if (tid_x() == 0) s[(int64_t)rb * ncb + cb] = sc;
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     float a[8];

@@ -23,8 +23,8 @@ __global__ __launch_bounds__(256) void stream_rw_kernel(const uint4* __restrict_
   const int64_t most = read_chunks > write_chunks ? read_chunks : write_chunks;
   constexpr int kStep = 256 * UNROLL;  // chunks per workgroup and step
   const int64_t steps = (most + kStep - 1) / kStep;
-  const int G = (int)gridDim.x;
-  int wg = (int)blockIdx.x;
+  const int G = (int)n_wg_x();
+  int wg = (int)wg_x();
   if (order == 2) {
     // workgroup i runs on XCD i % 8: give every XCD one contiguous eighth of the steps
     const int per = (G + 7) >> 3;
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void stream_rw_kernel(const uint4* __restrict_
   if (s1 > steps) s1 = steps;
   const int64_t ds = order == 0 ? G : 1;
   for (int64_t s = s0; s < s1; s += ds) {
-    const int64_t base = s * kStep + threadIdx.x;
+    const int64_t base = s * kStep + tid_x();
     uint4 v[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {

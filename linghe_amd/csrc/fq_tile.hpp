@@ -68,12 +68,12 @@ struct SubTile {
 };
 template <int RPT>
 __device__ __forceinline__ SubTile<RPT> sub_tile(int kc_shift) {
-  const int rg = threadIdx.x >> 4;
+  const int rg = tile_tid() >> 4;
   const int rgs = (kGroup / RPT) >> kc_shift;  // row groups per sub-tile
   SubTile<RPT> t;
   t.sub = __builtin_amdgcn_readfirstlane(rg / rgs);
   t.rgl = rg & (rgs - 1);
-  t.ws = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6) & ((rgs >> 2) - 1));
+  t.ws = __builtin_amdgcn_readfirstlane((int)(tile_tid() >> 6) & ((rgs >> 2) - 1));
   return t;
 }
 
@@ -179,7 +179,7 @@ __device__ __forceinline__ void quantize_tiles_impl(const float (&v)[NV][RPT][8]
                                                     TileShared<RPT, NV>& sh) {
   using Shape = TileShape<RPT>;
   static_assert(NV * kGroup <= Shape::kThreads, "one thread per column scale");
-  const int tid = threadIdx.x;
+  const int tid = tile_tid();
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int cg = tid & 15;
@@ -474,7 +474,7 @@ __device__ __forceinline__ ExpertShape expert_shape(int c, int ncb, int pad) {
 constexpr int kLookupSteps = 16;  // 64 experts per step: the counts of up to 1024 experts are fetched together
 __device__ __forceinline__ void load_counts(const void* counts, int is_i64, int n_experts, int base0, int steps,
                                             int (&cs)[kLookupSteps]) {
-  const int lane = threadIdx.x & 63;
+  const int lane = tile_tid() & 63;
 #pragma unroll
   for (int k = 0; k < kLookupSteps; ++k) {
     cs[k] = 0;

@@ -41,9 +41,9 @@ template <bool BATCHED>
 __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out_w, const BatchArgs& b,
                                                  int remap = 0) {
   TileGeom g;
-  int id = blockIdx.x;
+  int id = wg_x();
   if (remap == 1) {  // workgroup-uniform
-    const int G = (int)gridDim.x;
+    const int G = (int)n_wg_x();
     const int per = (G + 7) >> 3;
     const int xcd = id & 7, slot = id >> 3;
     // the first (G % 8, or 8) XCDs hold `per` tiles, the others one fewer
@@ -124,12 +124,12 @@ __device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g,
 // RPT rows x 8 bf16 columns of a row-major matrix; rows >= rows_valid read as 0
 // STREAM: loads carry the non-temporal hint (the tile is not read again).
 // SCALAR: the tile base, the same in every lane of a wave, is moved to scalar registers
-// rgl: the thread's row group (rows rgl*RPT ..): threadIdx.x >> 4 in an unpacked tile, the row
+// rgl: the thread's row group (rows rgl*RPT ..): tile_tid() >> 4 in an unpacked tile, the row
 // group inside the wave's sub-tile in a packed one (then base points at that sub-tile's columns)
 template <int RPT, bool STREAM = false, bool SCALAR = true>
 __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT],
                                           int rgl) {
-  const int cg = threadIdx.x & 15;
+  const int cg = tile_tid() & 15;
   // a tile spans at most 128 rows of at most 2^24 bytes (the widest input the entry
   // points accept), so lane offsets fit 32 bits
   const uint8_t* b = (const uint8_t*)base;
@@ -152,7 +152,7 @@ __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int 
 }
 template <int RPT, bool STREAM = false, bool SCALAR = true>
 __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT]) {
-  load_rows<RPT, STREAM, SCALAR>(base, ld, rows_valid, raw, (int)(threadIdx.x >> 4));
+  load_rows<RPT, STREAM, SCALAR>(base, ld, rows_valid, raw, (int)(tile_tid() >> 4));
 }
 
 // The part of a (possibly packed) tile this thread's wave works on, and how many of its rows exist

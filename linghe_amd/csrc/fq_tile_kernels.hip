@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
   __shared__ TileShared<RPT> sh;
   const TileGeom g = resolve_tile<true>(M, N / kGroup, N, batch);
   if (!g.valid) return;
-  const int cg = threadIdx.x & 15;
+  const int cg = tile_tid() & 15;
   const TilePart<RPT> tp = tile_part<RPT>(g);
   const int rg = tp.sl.rgl;
   // the 8 source rows of this thread: two 16-byte loads (regions start at multiples of 16 rows)
@@ -72,8 +72,8 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
     if (rg * RPT + s < tp.rows && (uint32_t)src[s] < (uint64_t)src_rows)
       raw[s] = load16<Policy::kLoadHintPermute>(col + (int64_t)src[s] * N);
   }
-  if (probs != nullptr && g.cb == 0 && threadIdx.x < kGroup) {
-    const int i = threadIdx.x;
+  if (probs != nullptr && g.cb == 0 && tile_tid() < kGroup) {
+    const int i = tile_tid();
     if (i < g.rows_store) {
       const int e = g.expert;
       float pv = 0.f;
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, N, tp.rows, r1, tp.sl.rgl);
   load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, N, tp.rows, r2, tp.sl.rgl);
   load_rows<RPT, LDNT>(gr + g.row0 * n + (int64_t)tp.cb * kGroup, n, tp.rows, rgd, tp.sl.rgl);
-  const int cg = threadIdx.x & 15;
+  const int cg = tile_tid() & 15;
   const int rg = tp.sl.rgl;
   float d[2][RPT][8];  // dx1, dx2
   float my_dw = 0.f;
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
 // dw[r] = sum_b part[r, b]  (fixed order), stored as fp32 or bf16
 __global__ __launch_bounds__(256) void rowsum_kernel(const float* __restrict__ part, void* __restrict__ dw,
                                                      int64_t M, int nb, int out_bf16) {
-  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t r = (int64_t)wg_x() * 256 + tile_tid();
   if (r >= M) return;
   float acc = 0.f;
   for (int b = 0; b < nb; ++b) acc += part[r * nb + b];
@@ -267,8 +267,8 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadRmsnorm) void rmsnorm_
   if (!g.valid) return;
   uint4 raw[RPT];
   load_rows<RPT, Policy::kLoadHintRmsnorm>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
-  const int cg = threadIdx.x & 15;
-  const int rg = threadIdx.x >> 4;
+  const int cg = tile_tid() & 15;
+  const int rg = tile_tid() >> 4;
   float gm[8];
   unpack8(*(const uint4*)(gamma + (int64_t)g.cb * kGroup + cg * 8), gm);
   float v[RPT][8];
