@@ -206,8 +206,8 @@ int fq_batched_swiglu_quant_fwd(const void* x, const void* weight, int weight_is
                                 int fp8_kind, void* stream);
 
 /* triton_batch_weighted_silu_and_block_quant_backward, linghe/utils/silu.py:1293-1393.
- * dw [M] in the weight's dtype; dw_partials fp32 [M, n/128] scratch (the
- * reference's dws). */
+ * dw [M] in the weight's dtype; dw_partials: M * n/128 floats of scratch (the
+ * reference's dws; what it holds afterwards is not part of the interface). */
 int fq_batched_swiglu_quant_bwd(const void* g, const void* x, const void* weight, int weight_is_bf16,
                                 const void* counts, int counts_is_i64, int n_experts, int64_t total_blocks,
                                 void* dq, float* ds, void* dw, void* dqt, float* dst, float* dw_partials,

@@ -217,7 +217,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   if constexpr (BATCHED) {
     if (cg < RPT) {
       const int i = rg * RPT + cg;
-      if (i < tp.rows) dw_part[(g.row0 + i) * nb + tp.cb] = my_dw;
+      if (i < tp.rows) dw_part[(int64_t)tp.cb * M + (g.row0 + i)] = my_dw;  // [nb, M]: a wave writes consecutive floats
     }
   }
   if constexpr (!BATCHED) {
@@ -230,23 +230,29 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
     // the single-matrix form takes M % 128 == 0 only (as the reference): no partial tile
     quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 2, false, true>(d, outs, sh);
   } else {
-    __shared__ TileShared<RPT> sh;
-    const TileOut o1[1] = {make_out(out, g, N, g.cb)};
-    const TileOut o2[1] = {make_out(out, g, N, nb + g.cb)};
-    const float (&dx1)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(d[0]);
-    const float (&dx2)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(d[1]);
-    quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 1, true>(dx1, o1, sh);
-    quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 1, false>(dx2, o2, sh);
+    // a full tile (most of them) goes the same way; a partial one, which may be packed, one tile after the other
+    __shared__ union { TileShared<RPT, 2> both; TileShared<RPT> one; } sh;
+    if (g.rows_store == kGroup) {
+      const TileOut outs[2] = {make_out(out, g, N, g.cb), make_out(out, g, N, nb + g.cb)};
+      quantize_tiles<KIND, ROUND, 2, RPT, NT, true, 2, false, true>(d, outs, sh.both);
+    } else {
+      const TileOut o1[1] = {make_out(out, g, N, g.cb)};
+      const TileOut o2[1] = {make_out(out, g, N, nb + g.cb)};
+      const float (&dx1)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(d[0]);
+      const float (&dx2)[1][RPT][8] = reinterpret_cast<const float (&)[1][RPT][8]>(d[1]);
+      quantize_tiles_impl<KIND, ROUND, 2, RPT, false, NT, true, 1, true>(dx1, o1, sh.one);
+      quantize_tiles_impl<KIND, ROUND, 2, RPT, false, NT, true, 1, false>(dx2, o2, sh.one);
+    }
   }
 }
 
-// dw[r] = sum_b part[r, b]  (fixed order), stored as fp32 or bf16
+// dw[r] = sum_b part[b, r]  (fixed order), stored as fp32 or bf16
 __global__ __launch_bounds__(256) void rowsum_kernel(const float* __restrict__ part, void* __restrict__ dw,
                                                      int64_t M, int nb, int out_bf16) {
   const int64_t r = (int64_t)wg_x() * 256 + tile_tid();
   if (r >= M) return;
   float acc = 0.f;
-  for (int b = 0; b < nb; ++b) acc += part[r * nb + b];
+  for (int b = 0; b < nb; ++b) acc += part[(int64_t)b * M + r];
   if (out_bf16) ((uint16_t*)dw)[r] = (uint16_t)(pack_bf16x2(acc, 0.f) & 0xffffu);
   else ((float*)dw)[r] = acc;
 }
