@@ -211,15 +211,25 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
     // one row in registers, the other waves cover its loads
     uint4 buf[NCHUNK];
     int parity = 0;
-    for (int64_t row = r0; row < r1; row += G) {
-      load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + row * n, n, buf);
+    // the first row's loads leave before gamma is waited for (see the fences below)
+    load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + r0 * n, n, buf);
+#pragma unroll
+    for (int k = 0; k < NCHUNK; ++k) fence_packed(gm[k]);
+    for (int64_t row = r0;;) {
       process(buf, row, parity);
       parity ^= 1;
+      row += G;
+      if (row >= r1) break;
+      load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + row * n, n, buf);
     }
     return;
   }
   uint4 bufA[NCHUNK], bufB[NCHUNK];
   load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + r0 * n, n, bufA);
+  // gamma is widened to fp32 once, before the loop; fenced here so that this happens (and gamma is
+  // waited for) after the first row's loads have left, not before (a wave has only M / 8192 rows)
+#pragma unroll
+  for (int k = 0; k < NCHUNK; ++k) fence_packed(gm[k]);
   for (int64_t row = r0; row < r1; row += 2 * G) {
     if (row + G < r1) load_row_clamped<T, NCHUNK, Policy::kLoadHintRows>(x + (row + G) * n, n, bufB);
     process(bufA, row, 0);
