@@ -111,6 +111,14 @@ struct RowWeight {
 __device__ __forceinline__ float load_weight(const RowWeight& w, int64_t r) {
   return w.is_bf16 ? as_f32((uint32_t)((const uint16_t*)w.w)[r] << 16) : ((const float*)w.w)[r];
 }
+// The same in two steps, so that several weights can be in flight together: the bits as loaded
+// (no arithmetic on them, hence no wait), widened where the weight is used.
+__device__ __forceinline__ uint32_t load_weight_bits(const RowWeight& w, int64_t r) {
+  return w.is_bf16 ? (uint32_t)((const uint16_t*)w.w)[r] : ((const uint32_t*)w.w)[r];
+}
+__device__ __forceinline__ float weight_from_bits(const RowWeight& w, uint32_t bits) {
+  return as_f32(bits << (w.is_bf16 ? 16 : 0));
+}
 
 // fp32 pair -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950)
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
