@@ -65,13 +65,19 @@ __global__ __launch_bounds__(256) void pad_permute_quant_kernel(const uint16_t* 
   }
   uint4 raw[RPT];
   const uint16_t* col = x + (int64_t)tp.cb * kGroup + cg * 8;
+  // Rows of the padding, and indices that do not name a source row, read as zero.  The eight loads
+  // carry no condition (such a row fetches source row 0, which exists, and is zeroed afterwards):
+  // behind a per-row branch the compiler waited for each gathered row before it asked for the
+  // next one, eight memory round trips in a row at the start of every tile.
+  bool live[RPT];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) {
-    raw[s] = make_uint4(0, 0, 0, 0);
-    // rows of the padding, and indices that do not name a source row, read as zero
-    if (rg * RPT + s < tp.rows && (uint32_t)src[s] < (uint64_t)src_rows)
-      raw[s] = load16<Policy::kLoadHintPermute>(col + (int64_t)src[s] * N);
+    live[s] = rg * RPT + s < tp.rows && (uint32_t)src[s] < (uint64_t)src_rows;
+    raw[s] = load16<Policy::kLoadHintPermute>(col + (int64_t)(live[s] ? src[s] : 0) * N);
   }
+#pragma unroll
+  for (int s = 0; s < RPT; ++s)
+    if (!live[s]) raw[s] = make_uint4(0, 0, 0, 0);
   if (probs != nullptr && g.cb == 0 && tile_tid() < kGroup) {
     const int i = tile_tid();
     if (i < g.rows_store) {
