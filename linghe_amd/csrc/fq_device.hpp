@@ -116,6 +116,18 @@ __device__ __forceinline__ float load_weight(const RowWeight& w, int64_t r) {
 __device__ __forceinline__ uint32_t load_weight_bits(const RowWeight& w, int64_t r) {
   return w.is_bf16 ? (uint32_t)((const uint16_t*)w.w)[r] : ((const uint32_t*)w.w)[r];
 }
+// R weights of rows r[0..R-1] (all of them valid addresses): one branch on the weight's type around
+// R straight loads, so that nothing waits between them
+template <int R>
+__device__ __forceinline__ void load_weight_bits(const RowWeight& w, const int64_t (&r)[R], uint32_t (&bits)[R]) {
+  if (w.is_bf16) {
+#pragma unroll
+    for (int s = 0; s < R; ++s) bits[s] = (uint32_t)((const uint16_t*)w.w)[r[s]];
+  } else {
+#pragma unroll
+    for (int s = 0; s < R; ++s) bits[s] = ((const uint32_t*)w.w)[r[s]];
+  }
+}
 __device__ __forceinline__ float weight_from_bits(const RowWeight& w, uint32_t bits) {
   return as_f32(bits << (w.is_bf16 ? 16 : 0));
 }

@@ -126,6 +126,12 @@ __device__ __forceinline__ TileOut make_out(const OutPtrs& p, const TileGeom& g,
 // SCALAR: the tile base, the same in every lane of a wave, is moved to scalar registers
 // rgl: the thread's row group (rows rgl*RPT ..): tile_tid() >> 4 in an unpacked tile, the row
 // group inside the wave's sub-tile in a packed one (then base points at that sub-tile's columns)
+// The loads carry no condition: a row beyond rows_valid fetches row 0 of the tile again (`base`
+// must be a valid address also when rows_valid is 0); the caller zeroes such rows with mask_rows
+// once every load of the tile has been issued.  With the loads
+// behind per-row branches, and a second, mask-free copy of them for full tiles, the compiler's
+// wait insertion turned conservative where the paths meet: the per-expert SwiGLU forward waited
+// for the whole x1 tile before it asked for x2.
 template <int RPT, bool STREAM = false, bool SCALAR = true>
 __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int rows_valid, uint4 (&raw)[RPT],
                                           int rgl) {
@@ -138,16 +144,21 @@ __device__ __forceinline__ void load_rows(const uint16_t* base, int64_t ld, int 
     b = (const uint8_t*)uniform64((int64_t)b);
     pitch = (uint32_t)uniform32((int)pitch);
   }
-  const uint32_t off0 = (uint32_t)(rgl * RPT) * pitch + (uint32_t)cg * 16u;
-  if (rows_valid == kGroup) {  // workgroup-uniform: no per-row masks
+  const uint32_t col = (uint32_t)cg * 16u;
 #pragma unroll
-    for (int s = 0; s < RPT; ++s) raw[s] = load16<STREAM>(b + (off0 + (uint32_t)s * pitch));
-  } else {
+  for (int s = 0; s < RPT; ++s) {
+    const int i = rgl * RPT + s;
+    raw[s] = load16<STREAM>(b + ((uint32_t)(i < rows_valid ? i : 0) * pitch + col));
+  }
+}
+// zero the rows that load_rows fetched from beyond rows_valid; called after ALL loads of a tile
+// have been issued (it has to wait for the rows it touches)
+template <int RPT>
+__device__ __forceinline__ void mask_rows(int rows_valid, uint4 (&raw)[RPT], int rgl) {
+  if (rows_valid != kGroup) {  // workgroup-uniform
 #pragma unroll
-    for (int s = 0; s < RPT; ++s) {
-      raw[s] = make_uint4(0, 0, 0, 0);
-      if (rgl * RPT + s < rows_valid) raw[s] = load16<STREAM>(b + (off0 + (uint32_t)s * pitch));
-    }
+    for (int s = 0; s < RPT; ++s)
+      if (rgl * RPT + s >= rows_valid) raw[s] = make_uint4(0, 0, 0, 0);
   }
 }
 template <int RPT, bool STREAM = false, bool SCALAR = true>
@@ -161,6 +172,7 @@ struct TilePart {
   SubTile<RPT> sl;
   int rows;  // rows of this wave's sub-tile that exist (0: the column block lies beyond the matrix)
   int cb;    // its 128-column block
+  int asub;  // column block inside the workgroup's run to LOAD from: sl.sub, or 0 when rows == 0 (a valid address)
 };
 template <int RPT>
 __device__ __forceinline__ TilePart<RPT> tile_part(const TileGeom& g) {
@@ -168,6 +180,7 @@ __device__ __forceinline__ TilePart<RPT> tile_part(const TileGeom& g) {
   p.sl = sub_tile<RPT>(g.kc_shift);
   p.rows = p.sl.sub < g.n_sub ? g.rows_valid : 0;
   p.cb = g.cb + p.sl.sub;
+  p.asub = p.sl.sub < g.n_sub ? p.sl.sub : 0;
   return p;
 }
 

@@ -26,7 +26,8 @@ void blockwise_quant_kernel(const uint16_t* __restrict__ x, OutPtrs out, int64_t
   constexpr int NT = BATCHED ? Policy::kStoreHintBlockwiseBatched : Policy::kStoreHintBlockwise;
   constexpr bool LEAN = BATCHED || Policy::kLeanBlockwise;
   const TilePart<RPT> tp = tile_part<RPT>(g);
-  load_rows<RPT, LDNT, LEAN>(x + g.row0 * N + (int64_t)tp.cb * kGroup, N, tp.rows, raw, tp.sl.rgl);
+  load_rows<RPT, LDNT, LEAN>(x + g.row0 * N + (int64_t)(g.cb + tp.asub) * kGroup, N, tp.rows, raw, tp.sl.rgl);
+  mask_rows<RPT>(tp.rows, raw, tp.sl.rgl);
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) unpack8(raw[s], v[s]);
@@ -125,16 +126,20 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd) void silu_qua
   // middle of the tile's critical path (four of them in the backward kernel, whose rows are fenced
   // apart: 85.2 -> 77.5 us without the weights at 65536 x 1024, 256 experts).
   uint32_t wbits[RPT];
+  if constexpr (WEIGHTED) {
+    // no per-row condition on the loads: a row beyond the end of the tile fetches the tile's first
+    // row's weight (a valid address) and counts as zero where it is used
+    int64_t wr[RPT];
 #pragma unroll
-  for (int s = 0; s < RPT; ++s) {
-    wbits[s] = 0;
-    if constexpr (WEIGHTED) {
-      const int i = rg * RPT + s;
-      if (i < tp.rows) wbits[s] = load_weight_bits(weight, g.row0 + i);
-    }
+    for (int s = 0; s < RPT; ++s) wr[s] = g.row0 + (rg * RPT + s < tp.rows ? rg * RPT + s : 0);
+    load_weight_bits<RPT>(weight, wr, wbits);
   }
-  load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, ld, tp.rows, r1, tp.sl.rgl);
-  load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, ld, tp.rows, r2, tp.sl.rgl);
+  load_rows<RPT, LDNT>(p + tp.asub * kGroup, ld, tp.rows, r1, tp.sl.rgl);
+  load_rows<RPT, LDNT>(p + n + tp.asub * kGroup, ld, tp.rows, r2, tp.sl.rgl);
+  if constexpr (!ALL_FULL) {
+    mask_rows<RPT>(tp.rows, r1, tp.sl.rgl);
+    mask_rows<RPT>(tp.rows, r2, tp.sl.rgl);
+  }
   // Every wave does the arithmetic, also one whose rows all lie beyond the last row of a partial tile
   // (its inputs read as zeros and give zeros): a branch around the arithmetic keeps the zero-filled results
   // and the packed inputs alive side by side and costs 13-20 registers (73 -> 60 in the per-expert form:
@@ -146,7 +151,7 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadSiluFwd) void silu_qua
       float a[8], b[8];
       unpack8(r1[s], a);
       unpack8(r2[s], b);
-      const float w = WEIGHTED ? weight_from_bits(weight, wbits[s]) : 1.0f;
+      const float w = !WEIGHTED ? 1.0f : rg * RPT + s < tp.rows ? weight_from_bits(weight, wbits[s]) : 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         float y = (sigmoid_f32(a[j]) * a[j]) * b[j];
@@ -182,17 +187,20 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
   if constexpr (!BATCHED) tp.rows = kGroup;  // single matrix: M % 128 == 0
   // row weights first (see the forward kernel)
   uint32_t wbits[RPT];
+  if constexpr (BATCHED) {
+    int64_t wr[RPT];
 #pragma unroll
-  for (int s = 0; s < RPT; ++s) {
-    wbits[s] = 0;
-    if constexpr (BATCHED) {
-      const int i = tp.sl.rgl * RPT + s;
-      if (i < tp.rows) wbits[s] = load_weight_bits(weight, g.row0 + i);
-    }
+    for (int s = 0; s < RPT; ++s) wr[s] = g.row0 + (tp.sl.rgl * RPT + s < tp.rows ? tp.sl.rgl * RPT + s : 0);
+    load_weight_bits<RPT>(weight, wr, wbits);
   }
-  load_rows<RPT, LDNT>(p + tp.sl.sub * kGroup, N, tp.rows, r1, tp.sl.rgl);
-  load_rows<RPT, LDNT>(p + n + tp.sl.sub * kGroup, N, tp.rows, r2, tp.sl.rgl);
-  load_rows<RPT, LDNT>(gr + g.row0 * n + (int64_t)tp.cb * kGroup, n, tp.rows, rgd, tp.sl.rgl);
+  load_rows<RPT, LDNT>(p + tp.asub * kGroup, N, tp.rows, r1, tp.sl.rgl);
+  load_rows<RPT, LDNT>(p + n + tp.asub * kGroup, N, tp.rows, r2, tp.sl.rgl);
+  load_rows<RPT, LDNT>(gr + g.row0 * n + (int64_t)(g.cb + tp.asub) * kGroup, n, tp.rows, rgd, tp.sl.rgl);
+  if constexpr (BATCHED) {
+    mask_rows<RPT>(tp.rows, r1, tp.sl.rgl);
+    mask_rows<RPT>(tp.rows, r2, tp.sl.rgl);
+    mask_rows<RPT>(tp.rows, rgd, tp.sl.rgl);
+  }
   const int cg = tile_tid() & 15;
   const int rg = tp.sl.rgl;
   float d[2][RPT][8];  // dx1, dx2
@@ -216,7 +224,7 @@ __global__ __launch_bounds__(512, 4) void silu_quant_bwd_kernel(const uint16_t* 
       unpack8(r1[s], a);
       unpack8(r2[s], b);
       unpack8(rgd[s], go);
-      const float w = BATCHED ? weight_from_bits(weight, wbits[s]) : 1.0f;
+      const float w = !BATCHED ? 1.0f : rg * RPT + s < tp.rows ? weight_from_bits(weight, wbits[s]) : 0.f;
       float dw = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -298,13 +306,20 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadRmsnorm) void rmsnorm_
   load_rows<RPT, Policy::kLoadHintRmsnorm>(x + g.row0 * n + (int64_t)g.cb * kGroup, n, g.rows_valid, raw);
   const int cg = tile_tid() & 15;
   const int rg = tile_tid() >> 4;
+  // every load of the tile is issued before the first of them is waited for: the statistic of a
+  // row beyond the end is fetched from the tile's first row (a valid address) and not used
+  const uint4 gmraw = *(const uint4*)(gamma + (int64_t)g.cb * kGroup + cg * 8);
+  float rs[RPT];
+#pragma unroll
+  for (int s = 0; s < RPT; ++s) rs[s] = rstd[g.row0 + (rg * RPT + s < g.rows_valid ? rg * RPT + s : 0)];
+  mask_rows<RPT>(g.rows_valid, raw, rg);
   float gm[8];
-  unpack8(*(const uint4*)(gamma + (int64_t)g.cb * kGroup + cg * 8), gm);
+  unpack8(gmraw, gm);
   float v[RPT][8];
 #pragma unroll
   for (int s = 0; s < RPT; ++s) {
     const int i = rg * RPT + s;
-    const float r = (i < g.rows_valid) ? rstd[g.row0 + i] : 0.f;
+    const float r = (i < g.rows_valid) ? rs[s] : 0.f;
     float a[8];
     unpack8(raw[s], a);
 #pragma unroll
