@@ -128,6 +128,18 @@ __device__ __forceinline__ void load_weight_bits(const RowWeight& w, const int64
     for (int s = 0; s < R; ++s) bits[s] = ((const uint32_t*)w.w)[r[s]];
   }
 }
+// The weight of a row that is the same in every lane of the wave (wave-per-row kernels): a scalar
+// load through the constant path, which neither queues behind the wave's vector loads nor counts
+// against their wait counter.  A bf16 weight is read as the aligned dword that holds it (inside
+// the array or, for the last element of an odd-length array, inside the same 4-byte word).
+__device__ __forceinline__ float load_weight_uniform(const RowWeight& w, int64_t r) {
+  typedef const __attribute__((address_space(4))) uint32_t* const_u32;
+  if (w.is_bf16) {
+    const uint32_t d = ((const_u32)(uintptr_t)w.w)[r >> 1];
+    return as_f32((r & 1) ? (d & 0xffff0000u) : (d << 16));
+  }
+  return as_f32(((const_u32)(uintptr_t)w.w)[r]);
+}
 __device__ __forceinline__ float weight_from_bits(const RowWeight& w, uint32_t bits) {
   return as_f32(bits << (w.is_bf16 ? 16 : 0));
 }

@@ -759,12 +759,14 @@ __global__ __launch_bounds__(64) void swiglu_fwd_rows_kernel(const uint16_t* __r
   for (int64_t row = wg_x(); row < M; row += n_wg_x()) {
     const uint16_t* p = x + row * 2 * (int64_t)n;
     float w = 1.0f;
-    if constexpr (WEIGHTED) w = load_weight(weight, row);
+    if constexpr (WEIGHTED) w = load_weight_uniform(weight, row);
     for (int c0 = 0; c0 < chunks; c0 += 256) {
       uint4 r1[4], r2[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        // unconditional loads: beyond the end of the row the last chunk is read again (never stored)
+        // No condition on loads or stores: beyond the end of the row a lane reads the row's last chunk
+        // again and stores the same result to the same place again.  (With the stores behind per-chunk
+        // branches the compiler waited for a step's stores before it issued the next step's loads.)
         const int c = c0 + u * 64 + lane;
         const int cc = c < chunks ? c : chunks - 1;
         r1[u] = ld16(p + cc * 8);
@@ -773,6 +775,7 @@ __global__ __launch_bounds__(64) void swiglu_fwd_rows_kernel(const uint16_t* __r
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int c = c0 + u * 64 + lane;
+        const int cc = c < chunks ? c : chunks - 1;
         float a[8], b[8], y[8];
         unpack8(r1[u], a);
         unpack8(r2[u], b);
@@ -781,7 +784,7 @@ __global__ __launch_bounds__(64) void swiglu_fwd_rows_kernel(const uint16_t* __r
           y[j] = (sigmoid_f32(a[j]) * a[j]) * b[j];
           if constexpr (WEIGHTED) y[j] = y[j] * w;
         }
-        if (c < chunks) st16(out + row * n + c * 8, pack8_bf16(y));
+        st16(out + row * n + cc * 8, pack8_bf16(y));
       }
     }
   }
@@ -799,46 +802,44 @@ __global__ __launch_bounds__(64) void swiglu_bwd_rows_kernel(const uint16_t* __r
     const uint16_t* gp = gr + row * (int64_t)n;
     uint16_t* o = dx + row * 2 * (int64_t)n;
     float w = 1.0f;
-    if constexpr (WEIGHTED) w = load_weight(weight, row);
+    if constexpr (WEIGHTED) w = load_weight_uniform(weight, row);
     float dws = 0.f;
     for (int c0 = 0; c0 < chunks; c0 += 128) {
       uint4 r1[2], r2[2], rg[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
+        // no condition on loads or stores (see the forward kernel); a repeated chunk adds nothing to dw
         const int c = c0 + u * 64 + lane;
-        r1[u] = make_uint4(0, 0, 0, 0);
-        r2[u] = make_uint4(0, 0, 0, 0);
-        rg[u] = make_uint4(0, 0, 0, 0);
-        if (c < chunks) {
-          r1[u] = ld16(p + c * 8);
-          r2[u] = ld16(p + n + c * 8);
-          rg[u] = ld16(gp + c * 8);
-        }
+        const int cc = c < chunks ? c : chunks - 1;
+        r1[u] = ld16(p + cc * 8);
+        r2[u] = ld16(p + n + cc * 8);
+        rg[u] = ld16(gp + cc * 8);
       }
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int c = c0 + u * 64 + lane;
+        const int cc = c < chunks ? c : chunks - 1;
         float a[8], b[8], go[8], d1[8], d2[8];
         unpack8(r1[u], a);
         unpack8(r2[u], b);
         unpack8(rg[u], go);
+        float part = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float sg = sigmoid_f32(a[j]);
           const float sx = sg * a[j];
           float gw = go[j];
           if constexpr (WEIGHTED) {
-            dws += go[j] * (sx * b[j]);
+            part += go[j] * (sx * b[j]);
             gw = go[j] * w;
           }
           const float h = gw * b[j];
           d2[j] = gw * sx;
           d1[j] = h * sg + ((h * a[j]) * (1.0f - sg)) * sg;
         }
-        if (c < chunks) {
-          st16(o + c * 8, pack8_bf16(d1));
-          st16(o + n + c * 8, pack8_bf16(d2));
-        }
+        if constexpr (WEIGHTED) dws += c < chunks ? part : 0.f;
+        st16(o + cc * 8, pack8_bf16(d1));
+        st16(o + n + cc * 8, pack8_bf16(d2));
       }
     }
     if constexpr (WEIGHTED) {
