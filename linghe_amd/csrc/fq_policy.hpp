@@ -69,6 +69,9 @@ struct Policy {
   static constexpr int kRowsPerThreadBlockwise = 8;
   static constexpr int kRowsPerThreadBlockwiseBatched = 4;
   static constexpr int kRowsPerThreadRmsnorm = 4;
+  // 1x128 groups per thread and step of the plain group quantiser (their loads are in flight together):
+  // 10.3 / 10.5 / 13.0 us with 1 / 2 / 4 at 8192 x 2048, where a thread has two groups in all
+  static constexpr int kGroupQuantUnroll = 1;
 
   // ---- the SwiGLU backwards widen row s of their packed inputs after row s-1 is done (fence_values):
   // without it the per-expert form needed 136 registers under its cap of 128 and spilled; with it (and no

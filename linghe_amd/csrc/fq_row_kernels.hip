@@ -529,22 +529,29 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t* __rest
   const int64_t g0 = ((int64_t)wg_x() * 256 + tid_x()) >> 4;
   const int64_t stride = ((int64_t)n_wg_x() * 256) >> 4;
   const int sub = tid_x() & 15;
-  const int64_t limit = (n_groups + stride - 1) / stride * stride;  // keep the 16 lanes of a row together
-  for (int64_t g = g0; g < limit; g += stride) {
-    const bool ok = g < n_groups;
-    uint4 raw = make_uint4(0, 0, 0, 0);
-    if (ok) raw = ld16(x + g * kGroup + sub * 8);
-    float a[8];
-    unpack8(raw, a);
-    float m = 0.f;
+  // kU groups per thread and step, their loads in flight together.  No condition on loads or stores: a
+  // group beyond the end repeats the last group (same result stored to the same place again).
+  constexpr int kU = Policy::kGroupQuantUnroll;
+  for (int64_t g = g0; g < n_groups; g += kU * stride) {
+    uint4 raw[kU];
+    int64_t gi[kU];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(a[j]));
-    m = row16_max(m);
-    const float sc = make_scale<KIND, ROUND>(m);
-    const uint2 pk = quantize8<KIND, ROUND>(a, make_quantum<ROUND>(sc));
-    if (ok) {
-      st8(q + g * kGroup + sub * 8, pk);
-      if (sub == 0) s[g] = sc;
+    for (int u = 0; u < kU; ++u) {
+      gi[u] = g + u * stride < n_groups ? g + u * stride : n_groups - 1;
+      raw[u] = ld16(x + gi[u] * kGroup + sub * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      float a[8];
+      unpack8(raw[u], a);
+      float m = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(a[j]));
+      m = row16_max(m);
+      const float sc = make_scale<KIND, ROUND>(m);
+      const uint2 pk = quantize8<KIND, ROUND>(a, make_quantum<ROUND>(sc));
+      st8(q + gi[u] * kGroup + sub * 8, pk);
+      if (sub == 0) s[gi[u]] = sc;
     }
   }
 }
