@@ -69,6 +69,9 @@ struct Policy {
   static constexpr int kRowsPerThreadBlockwise = 8;
   static constexpr int kRowsPerThreadBlockwiseBatched = 4;
   static constexpr int kRowsPerThreadRmsnorm = 4;
+  // the wide-row (four waves per row) RMSNorm + row-wise quant kernel loads the next row while it works on
+  // the current one (122 instead of 84 registers): 68.5 -> 65.5 us at 16384 x 7168
+  static constexpr bool kPrefetchRowQuantWide = true;
   // 1x128 groups per thread and step of the plain group quantiser (their loads are in flight together):
   // 10.3 / 10.5 / 13.0 us with 1 / 2 / 4 at 8192 x 2048, where a thread has two groups in all
   static constexpr int kGroupQuantUnroll = 1;

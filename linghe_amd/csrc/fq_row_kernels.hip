@@ -206,7 +206,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
     }
   };
 
-  if constexpr (OUT == 1) {
+  if constexpr (OUT == 1 && !(T == 256 && Policy::kPrefetchRowQuantWide)) {
     // the quantising form has enough arithmetic per row to want several waves per SIMD:
     // one row in registers, the other waves cover its loads
     uint4 buf[NCHUNK];
