@@ -72,6 +72,9 @@ struct Policy {
   // the wide-row (four waves per row) RMSNorm + row-wise quant kernel loads the next row while it works on
   // the current one (122 instead of 84 registers): 68.5 -> 65.5 us at 16384 x 7168
   static constexpr bool kPrefetchRowQuantWide = true;
+  // the same in the wide-row RMSNorm backward with one chunk per thread (2048 < n <= 4096: 70.4 -> 66.9 us at
+  // 16384 x 3072, 78.5 -> 76.4 at 16384 x 4096); with two chunks the second register set spills
+  static constexpr bool kPrefetchRowBwdWide = true;
   // 1x128 groups per thread and step of the plain group quantiser (their loads are in flight together):
   // 10.3 / 10.5 / 13.0 us with 1 / 2 / 4 at 8192 x 2048, where a thread has two groups in all
   static constexpr int kGroupQuantUnroll = 1;

@@ -325,14 +325,14 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
   // that two 512-thread workgroups fit a CU and cover each other's waits.  Prefetching
   // the next row's packed data into a second register set spills (142 -> 198 us at
   // 16384 x 7168 with 512 threads, 155 -> 179 us with 256 threads and four chunks).
-  int parity = 0;
-  for (int64_t row = wg_x(); row < M; row += G) {
-    uint4 rx[NCHUNK], rg[NCHUNK];
+  auto fetch = [&](int64_t row, uint4 (&rx)[NCHUNK], uint4 (&rg)[NCHUNK]) {
 #pragma unroll
     for (int k = 0; k < NCHUNK; ++k) {
       rx[k] = load16<Policy::kLoadHintRows>(x + row * n + cidx[k] * 8);
       rg[k] = load16<Policy::kLoadHintRows>(dy + row * n + cidx[k] * 8);
     }
+  };
+  auto process = [&](int64_t row, uint4 (&rx)[NCHUNK], uint4 (&rg)[NCHUNK], int parity) {
     double ss = 0.0;
     float dot = 0.f;
 #pragma unroll
@@ -353,7 +353,6 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
     } else {
       block_sum2<T>(ss, dot, sh, parity);
     }
-    parity ^= 1;
     forget<NCHUNK>(rx);
     forget<NCHUNK>(rg);
     float r;
@@ -371,6 +370,27 @@ __global__ __launch_bounds__(T, 4) void rmsnorm_bwd_kernel(const uint16_t* __res
         acc[k][j] = __builtin_fmaf(a[j] * g[j], r, acc[k][j]);  // dgamma: one rounding fewer per term
       }
       if (live[k]) st16(dx + row * n + cidx[k] * 8, pack8_bf16(o));
+    }
+  };
+  if constexpr (Policy::kPrefetchRowBwdWide && NCHUNK == 1) {
+    uint4 xa[NCHUNK], ga[NCHUNK], xb[NCHUNK], gb[NCHUNK];
+    const int64_t r0 = wg_x();
+    if (r0 < M) fetch(r0, xa, ga);
+    for (int64_t row = r0; row < M; row += 2 * G) {
+      if (row + G < M) fetch(row + G, xb, gb);
+      process(row, xa, ga, 0);
+      if (row + G < M) {
+        if (row + 2 * G < M) fetch(row + 2 * G, xa, ga);
+        process(row + G, xb, gb, 1);
+      }
+    }
+  } else {
+    int parity = 0;
+    for (int64_t row = wg_x(); row < M; row += G) {
+      uint4 rx[NCHUNK], rg[NCHUNK];
+      fetch(row, rx, rg);
+      process(row, rx, rg, parity);
+      parity ^= 1;
     }
   }
   // every workgroup writes its (possibly zero) partial: the reduction reads all of them
