@@ -108,16 +108,9 @@ struct RowWeight {
   const void* w;
   int is_bf16;
 };
-__device__ __forceinline__ float load_weight(const RowWeight& w, int64_t r) {
-  return w.is_bf16 ? as_f32((uint32_t)((const uint16_t*)w.w)[r] << 16) : ((const float*)w.w)[r];
-}
-// The same in two steps, so that several weights can be in flight together: the bits as loaded
-// (no arithmetic on them, hence no wait), widened where the weight is used.
-__device__ __forceinline__ uint32_t load_weight_bits(const RowWeight& w, int64_t r) {
-  return w.is_bf16 ? (uint32_t)((const uint16_t*)w.w)[r] : ((const uint32_t*)w.w)[r];
-}
-// R weights of rows r[0..R-1] (all of them valid addresses): one branch on the weight's type around
-// R straight loads, so that nothing waits between them
+// R weights of rows r[0..R-1] (all of them valid addresses) as loaded, to be widened where they are
+// used (weight_from_bits): no arithmetic on them here, hence no wait, and one branch on the weight's
+// type around R straight loads, so that they are in flight together
 template <int R>
 __device__ __forceinline__ void load_weight_bits(const RowWeight& w, const int64_t (&r)[R], uint32_t (&bits)[R]) {
   if (w.is_bf16) {
@@ -130,13 +123,14 @@ __device__ __forceinline__ void load_weight_bits(const RowWeight& w, const int64
 }
 // The weight of a row that is the same in every lane of the wave (wave-per-row kernels): a scalar
 // load through the constant path, which neither queues behind the wave's vector loads nor counts
-// against their wait counter.  A bf16 weight is read as the aligned dword that holds it (inside
-// the array or, for the last element of an odd-length array, inside the same 4-byte word).
+// against their wait counter.  A bf16 weight is read as the aligned 4-byte word that holds it (the
+// word may reach two bytes beyond either end of the array, never beyond the word of a valid element).
 __device__ __forceinline__ float load_weight_uniform(const RowWeight& w, int64_t r) {
   typedef const __attribute__((address_space(4))) uint32_t* const_u32;
   if (w.is_bf16) {
-    const uint32_t d = ((const_u32)(uintptr_t)w.w)[r >> 1];
-    return as_f32((r & 1) ? (d & 0xffff0000u) : (d << 16));
+    const uintptr_t at = (uintptr_t)w.w + 2 * (uintptr_t)r;  // the array may start on an odd element of its storage
+    const uint32_t d = *(const_u32)(at & ~(uintptr_t)3);
+    return as_f32((at & 2) ? (d & 0xffff0000u) : (d << 16));
   }
   return as_f32(((const_u32)(uintptr_t)w.w)[r]);
 }

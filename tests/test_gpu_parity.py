@@ -417,6 +417,32 @@ def test_weighted_silu(gpu, M, N, coef, wdtype):
                                    atol=tol * max(float(dw_ref.abs().max()), 1e-30))
 
 
+@pytest.mark.parametrize("offset", [1, 2, 3])
+def test_weighted_silu_bf16_weight_view(gpu, offset):
+    """A bf16 weight that starts on an odd element of its storage (a slice of a longer vector): the row
+    kernels read the weight as the aligned 4-byte word that holds it, so every alignment is tried."""
+    from linghe_amd.utils.silu import triton_weighted_silu_backward as bwd, triton_weighted_silu_forward as fwd
+
+    M, N = 257, 512
+    announce("weighted silu bf16, weight view at element", offset)
+    g = gen(47)
+    x = randn_bf16(g, M, N)
+    dy = randn_bf16(g, M, N // 2)
+    w = torch.randn(M, 1, generator=g).to(torch.bfloat16)
+    store = torch.zeros(M + 8, 1, dtype=torch.bfloat16, device=gpu)
+    wd = store[offset:offset + M]
+    wd.copy_(w)
+    assert wd.data_ptr() == store.data_ptr() + 2 * offset and wd.is_contiguous()
+    xd, dyd = _dev(x, gpu), _dev(dy, gpu)
+    y = fwd(xd, wd)
+    dx, dw = bwd(dyd, xd, wd)
+    torch.cuda.synchronize()
+    check_bf16("wsilu.view.y", O.weighted_silu_forward(x, w.float()), y)
+    dx_ref, dw_ref = O.weighted_silu_backward(dy, x, w.float())
+    check_bf16("wsilu.view.dx", dx_ref, dx)
+    torch.testing.assert_close(dw.cpu().float(), dw_ref.float(), rtol=2e-2, atol=2e-2 * float(dw_ref.abs().max()))
+
+
 @pytest.mark.parametrize("M,N", [(8192, 4096), (128, 128), (256, 1536)])
 @pytest.mark.parametrize("round_scale", [True, False])
 def test_block_quant(gpu, M, N, round_scale):
