@@ -831,10 +831,11 @@ __global__ __launch_bounds__(64) void swiglu_bwd_rows_kernel(const uint16_t* __r
     float w = 1.0f;
     if constexpr (WEIGHTED) w = load_weight_uniform(weight, row);
     float dws = 0.f;
-    for (int c0 = 0; c0 < chunks; c0 += 128) {
-      uint4 r1[2], r2[2], rg[2];
+    constexpr int kU = Policy::kSwigluBwdRowsUnroll;  // 16-byte chunks per lane, matrix and step
+    for (int c0 = 0; c0 < chunks; c0 += 64 * kU) {
+      uint4 r1[kU], r2[kU], rg[kU];
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < kU; ++u) {
         // no condition on loads or stores (see the forward kernel); a repeated chunk adds nothing to dw
         const int c = c0 + u * 64 + lane;
         const int cc = c < chunks ? c : chunks - 1;
@@ -843,7 +844,7 @@ __global__ __launch_bounds__(64) void swiglu_bwd_rows_kernel(const uint16_t* __r
         rg[u] = ld16(gp + cc * 8);
       }
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < kU; ++u) {
         const int c = c0 + u * 64 + lane;
         const int cc = c < chunks ? c : chunks - 1;
         float a[8], b[8], go[8], d1[8], d2[8];
