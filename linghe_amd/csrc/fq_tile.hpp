@@ -472,15 +472,20 @@ __device__ __forceinline__ ExpertShape expert_shape(int c, int ncb, int pad) {
 }
 
 constexpr int kLookupSteps = 16;  // 64 experts per step: the counts of up to 1024 experts are fetched together
+// No condition on the loads and one code path for both count types: a lane beyond the last expert
+// fetches the last expert's count (the caller takes it as 0), an int64 count is read as its low half
+// (little endian; a count is a number of rows and fits 31 bits).
 __device__ __forceinline__ void load_counts(const void* counts, int is_i64, int n_experts, int base0, int steps,
                                             int (&cs)[kLookupSteps]) {
   const int lane = tile_tid() & 63;
+  const int shift = is_i64 ? 3 : 2;
+  const uint8_t* base = (const uint8_t*)counts;
 #pragma unroll
   for (int k = 0; k < kLookupSteps; ++k) {
     cs[k] = 0;
     if (k < steps) {
       const int e = base0 + k * 64 + lane;
-      if (e < n_experts) cs[k] = load_count(counts, is_i64, e);
+      cs[k] = *(const int*)(base + ((int64_t)(e < n_experts ? e : n_experts - 1) << shift));  // masked by the caller
     }
   }
 }
@@ -524,7 +529,7 @@ __device__ __forceinline__ ExpertTile find_expert_tile(const void* counts, int i
     for (int k = 0; k < kSteps; ++k) {
       if (k < steps) {
         const int base = base0 + k * 64;
-        const int c = cs[k];
+        const int c = base + (int)(tile_tid() & 63) < n_experts ? cs[k] : 0;
         const ExpertShape es = expert_shape(c, ncb, pad);
         const int pc = es.pc, nb = es.nb, shift = es.shift, nw = es.nw;
         const int rows = wave_inclusive_scan(pc);
