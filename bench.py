@@ -653,6 +653,7 @@ def time_cpu(case):
 STREAM_VARIANTS = [
     (4, 16384, 0, 0, 0), (4, 16384, 0, 1, 1),            # the plain form, without and with the hints
     (8, 2048, 0, 1, 1), (8, 0, 0, 1, 1), (8, 0, 1, 1, 1), (8, 0, 0, 1, 0), (8, 2048, 1, 1, 0),
+    (8, 2048, 0, 1, 0), (8, 0, 1, 1, 0),                 # the other two of the best four on a 2:1 read:write mix
     (4, 0, 0, 1, 1), (4, 512, 0, 1, 1), (16, 0, 0, 1, 1),
 ]
 
