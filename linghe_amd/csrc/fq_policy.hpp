@@ -75,6 +75,9 @@ struct Policy {
   // the wide-row (four waves per row) RMSNorm + row-wise quant kernel loads the next row while it works on
   // the current one (122 instead of 84 registers): 68.5 -> 65.5 us at 16384 x 7168
   static constexpr bool kPrefetchRowQuantWide = true;
+  // workgroups per CU of that kernel's launch (it holds four at 122 registers): 64.0 / 65.4 / 64.8 / 64.6 /
+  // 68.0 us with 4 / 5 / 6 / 8 / 12 at 16384 x 7168
+  static constexpr int kRowQuantWideWgsPerCu = 4;
   // the same in the wide-row RMSNorm backward with one chunk per thread (2048 < n <= 4096: 70.4 -> 66.9 us at
   // 16384 x 3072, 78.5 -> 76.4 at 16384 x 4096); with two chunks the second register set spills
   static constexpr bool kPrefetchRowBwdWide = true;

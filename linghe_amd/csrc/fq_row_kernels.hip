@@ -622,7 +622,7 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
   } else if (n > 2048) {
     // wide rows, quantising form: four waves per row (a wave per row needs up to ~230 registers)
     int64_t wg4 = M;
-    if (wg4 > 256 * 8) wg4 = 256 * 8;
+    if (wg4 > 256 * Policy::kRowQuantWideWgsPerCu) wg4 = 256 * Policy::kRowQuantWideWgsPerCu;
     const dim3 grid4((unsigned)wg4);
     const int nc4 = (n / 8 + 255) / 256;
 #define FQ_LAUNCH_FWD4(NC, KINDV, ROUNDV)                                                                      \
