@@ -654,6 +654,7 @@ STREAM_VARIANTS = [
     (4, 16384, 0, 0, 0), (4, 16384, 0, 1, 1),            # the plain form, without and with the hints
     (8, 2048, 0, 1, 1), (8, 0, 0, 1, 1), (8, 0, 1, 1, 1), (8, 0, 0, 1, 0), (8, 2048, 1, 1, 0),
     (8, 2048, 0, 1, 0), (8, 0, 1, 1, 0),                 # the other two of the best four on a 2:1 read:write mix
+    (4, 0, 0, 1, 0),                                     # the best on the SwiGLU backward's mix
     (4, 0, 0, 1, 1), (4, 512, 0, 1, 1), (16, 0, 0, 1, 1),
 ]
 
@@ -690,13 +691,15 @@ def stream_ceiling(case, dev, stream, steps, warmup, repeats):
 
 
 def stream_sweep(dev, stream, steps, warmup, repeats):
-    """Every variant of the no-work kernel on the byte counts of cfg1, cfg2 and cfg5a (read MB, write MB),
+    """Every variant of the no-work kernel on the byte counts of cfg1, cfg2, cfg4 and cfg5a (read MB, write MB),
     cold buffers: a markdown table on stdout (the basis of STREAM_VARIANTS)."""
     from linghe_amd import configs
     sizes = [("cfg1", configs.rw_rmsnorm_quant(8192, 2048, 2)), ("cfg2", configs.rw_swiglu_fwd(8192, 2048, 2)),
-             ("cfg5a", configs.rw_rmsnorm_bwd(16384, 7168))]
+             ("cfg4", configs.rw_swiglu_bwd(8192, 2048)), ("cfg5a", configs.rw_rmsnorm_bwd(16384, 7168))]
     variants = [(c, w, o, l, st) for c in (4, 8, 16) for w in (256, 512, 1024, 2048, 0) for o in (0, 1, 2)
                 for l in (0, 1) for st in (0, 1)]
+    # order 3: the access pattern of the tile kernels (steps are tiles of 256-byte row segments)
+    variants += [(c, w, 3, l, st) for c in (4, 8, 16) for w in (2048, 0) for l in (0, 1) for st in (0, 1)]
     variants.insert(0, (4, 16384, 0, 0, 0))
     variants.insert(1, (4, 16384, 0, 1, 1))
     cols = {}

@@ -62,7 +62,9 @@ int fq_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_b
 /* The same kernel in its variants (no counterpart in the reference either): chunks_per_lane = 16-byte
  * chunks in flight per lane (4, 8 or 16); workgroups = how many to launch (0: one step of
  * 256 * chunks_per_lane chunks per workgroup, else each walks several); order 0 = interleaved steps,
- * 1 = one contiguous run per workgroup, 2 = the same with one contiguous eighth of the buffers per XCD;
+ * 1 = one contiguous run per workgroup, 2 = the same with one contiguous eighth of the buffers per XCD,
+ * 3 = interleaved steps shaped as the tile kernels' accesses (a step is 16 * chunks_per_lane rows x 256 bytes
+ * of a matrix with 4096-byte rows);
  * nt_loads / nt_stores put the streaming hint on loads / stores.  fq_stream_rw is
  * (4, 16384, 0, nontemporal, nontemporal).  The measured ceiling is the fastest variant. */
 int fq_stream_rw_variant(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,

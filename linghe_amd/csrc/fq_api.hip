@@ -74,8 +74,8 @@ int fq_stream_rw_variant(const void* src, int64_t read_bytes, void* dst, int64_t
              FQ_ERR_ARG, "%s: NULL or misaligned pointer", fn);
   FQ_REQUIRE(chunks_per_lane == 4 || chunks_per_lane == 8 || chunks_per_lane == 16, FQ_ERR_ARG,
              "%s: chunks_per_lane must be 4, 8 or 16", fn);
-  FQ_REQUIRE(order >= 0 && order <= 2 && workgroups >= 0 && workgroups <= (1 << 24), FQ_ERR_ARG,
-             "%s: order must be 0, 1 or 2 and workgroups 0 .. 2^24", fn);
+  FQ_REQUIRE(order >= 0 && order <= 3 && workgroups >= 0 && workgroups <= (1 << 24), FQ_ERR_ARG,
+             "%s: order must be 0 .. 3 and workgroups 0 .. 2^24", fn);
   return check_launch(fq::launch_stream_rw(src, read_bytes, dst, write_bytes, sink, chunks_per_lane, workgroups, order,
                                            nt_loads != 0, nt_stores != 0, (hipStream_t)stream),
                       fn);

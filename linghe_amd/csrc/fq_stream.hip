@@ -36,24 +36,39 @@ __global__ __launch_bounds__(256) void stream_rw_kernel(const uint4* __restrict_
   // order 0: workgroup wg takes the steps wg, wg + G, wg + 2G, ... (at any time the grid works on one
   // contiguous window of the buffers); order 1 / 2: a contiguous run of per_wg steps per workgroup
   const int64_t per_wg = (steps + G - 1) / G;
-  int64_t s0 = order == 0 ? wg : (int64_t)wg * per_wg;
-  int64_t s1 = order == 0 ? steps : s0 + per_wg;
+  const bool strided = order == 0 || order == 3;
+  int64_t s0 = strided ? wg : (int64_t)wg * per_wg;
+  int64_t s1 = strided ? steps : s0 + per_wg;
   if (s1 > steps) s1 = steps;
-  const int64_t ds = order == 0 ? G : 1;
+  const int64_t ds = strided ? G : 1;
+  // order 3: a step is a TILE of 16 * UNROLL rows x 256 bytes of a matrix with 4096-byte rows (the access
+  // pattern of the 128 x 128 tile kernels: 16 lanes per 256-byte row segment), steps interleaved over the
+  // workgroups as in order 0; the tail that does not fill a block of rows is walked linearly
+  constexpr int kRowChunks = 256;                        // 16-byte chunks per matrix row
+  constexpr int64_t kBlockChunks = (int64_t)16 * UNROLL * kRowChunks;  // chunks per block of rows = 16 steps
   for (int64_t s = s0; s < s1; s += ds) {
     const int64_t base = s * kStep + tid_x();
+    int64_t idx[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) idx[u] = base + u * 256;
+    if (order == 3) {
+      const int64_t rb = s >> 4;
+      if ((rb + 1) * kBlockChunks <= most) {
+        const int cb = (int)(s & 15), row = ((int)tid_x() >> 4) * UNROLL, cgp = (int)tid_x() & 15;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) idx[u] = rb * kBlockChunks + (int64_t)(row + u) * kRowChunks + cb * 16 + cgp;
+      }
+    }
     uint4 v[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t i = base + u * 256;
-      v[u] = make_uint4((uint32_t)i, 0, 0, 0);
-      if (i < read_chunks) v[u] = load16<NT_LOAD>(src + i);
+      v[u] = make_uint4((uint32_t)idx[u], 0, 0, 0);
+      if (idx[u] < read_chunks) v[u] = load16<NT_LOAD>(src + idx[u]);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t i = base + u * 256;
       acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w;
-      if (i < write_chunks) store16<NT_STORE>(dst + i, v[u]);
+      if (idx[u] < write_chunks) store16<NT_STORE>(dst + idx[u], v[u]);
     }
   }
   // keeps the loads alive when nothing is written; never true for the all-zero or small-integer data of the bench
@@ -61,7 +76,8 @@ __global__ __launch_bounds__(256) void stream_rw_kernel(const uint4* __restrict_
 }
 
 // chunks_per_lane: 4, 8 or 16.  workgroups: how many to launch; 0 = one step per workgroup.
-// order: 0 interleaved steps, 1 a contiguous run per workgroup, 2 the same with one contiguous eighth per XCD.
+// order: 0 interleaved steps, 1 a contiguous run per workgroup, 2 the same with one contiguous eighth per XCD,
+// 3 interleaved steps that are tiles of 16 * chunks_per_lane rows x 256 bytes of a matrix with 4096-byte rows.
 hipError_t launch_stream_rw(const void* src, int64_t read_bytes, void* dst, int64_t write_bytes, void* sink,
                             int chunks_per_lane, int64_t workgroups, int order, int nt_loads,
                             int nt_stores, hipStream_t stream) {
@@ -69,7 +85,7 @@ hipError_t launch_stream_rw(const void* src, int64_t read_bytes, void* dst, int6
   const int64_t most = rc > wc ? rc : wc;
   if (most == 0) return hipSuccess;
   if (chunks_per_lane != 4 && chunks_per_lane != 8 && chunks_per_lane != 16) return hipErrorInvalidValue;
-  if (order < 0 || order > 2) return hipErrorInvalidValue;
+  if (order < 0 || order > 3) return hipErrorInvalidValue;
   const int64_t steps = (most + 256 * chunks_per_lane - 1) / (256 * chunks_per_lane);
   int64_t wgs = workgroups <= 0 || workgroups > steps ? steps : workgroups;
   if (wgs > (1 << 30)) return hipErrorInvalidValue;

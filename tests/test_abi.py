@@ -84,7 +84,7 @@ def test_c_side_validation_without_gpu():
     assert L.fq_pack_router_weight(None, 0, None, 2048, 256, None) == -1
     assert L.fq_rmsnorm_router_quant_fwd_packed(None, None, None, 0, None, None, None, None, None, 128, 2048, 100,
                                                 1e-6, 0, 0, None) == -2
-    # the no-work kernel's variants: chunks per lane 4 / 8 / 16 only, order 0..2
+    # the no-work kernel's variants: chunks per lane 4 / 8 / 16 only, order 0..3
     assert L.fq_stream_rw_variant(None, 0, None, 0, None, 4, 0, 0, 0, 0, None) == -1          # no sink
     assert L.fq_stream_rw_variant(None, 16, None, 0, None, 5, 0, 0, 0, 0, None) == -1
     assert L.fq_stream_rw_variant(None, 24, None, 0, None, 4, 0, 0, 0, 0, None) == -2         # not a multiple of 16
