@@ -69,6 +69,7 @@ struct Policy {
   static constexpr int kRowsPerThreadBlockwise = 8;
   static constexpr int kRowsPerThreadBlockwiseBatched = 4;
   static constexpr int kRowsPerThreadRmsnorm = 4;
+  static constexpr bool kStartPriorityRmsnorm = true;
   // 16-byte chunks per lane, matrix and step in the bf16 SwiGLU backward (three matrices are read):
   // 29.0 / 30.4 / 28.7 / 35.5 us with 2 / 3 / 4 / 8 at 8192 x 4096
   static constexpr int kSwigluBwdRowsUnroll = 4;
