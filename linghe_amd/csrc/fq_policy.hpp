@@ -69,6 +69,9 @@ struct Policy {
   static constexpr int kRowsPerThreadBlockwise = 8;
   static constexpr int kRowsPerThreadBlockwiseBatched = 4;
   static constexpr int kRowsPerThreadRmsnorm = 4;
+  // waves (one row each) per workgroup of the statistic pass: 18.10 / 18.00 / 18.00 / 18.04 us at 8192 x 2048 and
+  // 107.8 / 108.0 / 107.4 / 107.6 at 16384 x 7168 with 1 / 2 / 4 / 8
+  static constexpr int kRowstatWaves = 4;
   static constexpr bool kStartPriorityRmsnorm = true;
   // 16-byte chunks per lane, matrix and step in the bf16 SwiGLU backward (three matrices are read):
   // 29.0 / 30.4 / 28.7 / 35.5 us with 2 / 3 / 4 / 8 at 8192 x 4096

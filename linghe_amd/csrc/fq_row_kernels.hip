@@ -250,15 +250,16 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
 // columns, 8 beyond.  The loads carry no per-lane condition: a chunk beyond the end of the row
 // reads the row's last chunk again and counts as zero.
 template <int U>
-__global__ __launch_bounds__(64) void rowstat_kernel(const uint16_t* __restrict__ x, float* __restrict__ rstd,
+__global__ __launch_bounds__(64 * Policy::kRowstatWaves) void rowstat_kernel(const uint16_t* __restrict__ x, float* __restrict__ rstd,
                                                      int64_t M, int n, float eps) {
-  const int lane = tid_x();
+  constexpr int kW = Policy::kRowstatWaves;  // waves (rows) per workgroup
+  const int lane = tid_x() & 63;
   const int chunks = n >> 3;
   // Rows are taken from the END of the matrix backwards.  The tile kernel that follows
   // walks the matrix forwards, so it starts with the rows this kernel read last, which
   // are the ones still in the last-level cache: for an input about the size of that
   // cache roughly half of the second read never reaches HBM.
-  for (int64_t k = wg_x(); k < M; k += n_wg_x()) {
+  for (int64_t k = (int64_t)wg_x() * kW + (tid_x() >> 6); k < M; k += (int64_t)n_wg_x() * kW) {
     const int64_t row = M - 1 - k;
     const uint4* p = (const uint4*)(x + row * n);
     double ss = 0.0;
@@ -615,8 +616,9 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
                                    scale, rstd, M, n, eps, rows_per_wg);)
   // quant: 0 = bf16 output, 1 = fp8 codes + scales, 2 = statistic only (its own kernel)
   if (quant == 2) {
-    if (n <= 2048) hipLaunchKernelGGL(rowstat_kernel<4>, grid, dim3(64), 0, stream, (const uint16_t*)x, rstd, M, n, eps);
-    else hipLaunchKernelGGL(rowstat_kernel<8>, grid, dim3(64), 0, stream, (const uint16_t*)x, rstd, M, n, eps);
+    const dim3 sgrid((unsigned)((wgs + Policy::kRowstatWaves - 1) / Policy::kRowstatWaves)), sblock(64 * Policy::kRowstatWaves);
+    if (n <= 2048) hipLaunchKernelGGL(rowstat_kernel<4>, sgrid, sblock, 0, stream, (const uint16_t*)x, rstd, M, n, eps);
+    else hipLaunchKernelGGL(rowstat_kernel<8>, sgrid, sblock, 0, stream, (const uint16_t*)x, rstd, M, n, eps);
   } else if (!quant) {
     if (reuse_rstd) { FQ_LAUNCH_FWD(true, 0, kE4M3, false) } else { FQ_LAUNCH_FWD(false, 0, kE4M3, false) }
   } else if (n > 2048) {
