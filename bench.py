@@ -198,7 +198,17 @@ def build_cases(names, dev):
     add("cfg2_mode1", build=lambda: swiglu_fwd_case("cfg2_mode1", False, 1))
 
     # ---------------------------------------------------------------- cfg3 (+ backward)
-    def batched_case(backward):
+    def expert_plan(cnt, counts):
+        """the per-expert tile plan of a set of counts (table, shape), built once outside the timed region"""
+        import ctypes
+        host = (ctypes.c_int64 * len(counts))(*counts)
+        shape = (ctypes.c_int64 * 4)()
+        _lib.check(L.fq_expert_plan_shape(host, len(counts), shape))
+        table = torch.empty((max(int(L.fq_expert_plan_bytes(shape)), 16),), device=dev, dtype=torch.uint8)
+        _lib.check(L.fq_build_expert_plan(_p(cnt), 0, len(counts), shape, _p(table), stream))
+        return table, shape
+
+    def batched_case(backward, planned=False):
         d = lazy.setdefault("cfg3", configs.cfg3_batched_swiglu())
         x_cpu, w_cpu, counts, dy_cpu = d["x"], d["weight"], d["counts"], d["dy"]
         M, N = x_cpu.shape
@@ -206,6 +216,7 @@ def build_cases(names, dev):
         E = len(counts)
         blocks = sum((c + 127) // 128 for c in counts)
         cnt = torch.tensor(counts, dtype=torch.int32, device=dev)
+        plan, pshape = expert_plan(cnt, counts) if planned else (None, None)
         W = N if backward else n
 
         def make_set():
@@ -217,16 +228,21 @@ def build_cases(names, dev):
                 s["dy"] = dy_cpu.to(dev)
                 s["dw"] = torch.empty((M, 1), device=dev, dtype=torch.float32)
                 s["dws"] = torch.empty((M, n // 128), device=dev, dtype=torch.float32)
-                s["args"] = (_p(s["dy"]), _p(s["x"]), _p(s["w"]), 0, _p(cnt), 0, E, blocks, _p(s["q"]), _p(s["s"]),
-                             _p(s["dw"]), _p(s["qt"]), _p(s["st"]), _p(s["dws"]), M, n, 0, _lib.FQ_E4M3, stream)
+                src = (_p(plan), pshape) if planned else (_p(cnt), 0, E, blocks)
+                s["args"] = (_p(s["dy"]), _p(s["x"]), _p(s["w"]), 0) + src + (
+                    _p(s["q"]), _p(s["s"]), _p(s["dw"]), _p(s["qt"]), _p(s["st"]), _p(s["dws"]), M, n, 0,
+                    _lib.FQ_E4M3, stream)
             else:
-                s["args"] = (_p(s["x"]), _p(s["w"]), 0, _p(cnt), 0, E, blocks, _p(s["q"]), _p(s["s"]), _p(s["qt"]),
-                             _p(s["st"]), M, n, 0, 2, _lib.FQ_E4M3, stream)
+                src = (_p(plan), pshape) if planned else (_p(cnt), 0, E, blocks)
+                s["args"] = (_p(s["x"]), _p(s["w"]), 0) + src + (
+                    _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, n, 0, 2, _lib.FQ_E4M3, stream)
             return s
 
         if backward:
+            bwd_fn = L.fq_batched_swiglu_quant_bwd_planned if planned else L.fq_batched_swiglu_quant_bwd
+
             def launch(s):
-                _lib.check(L.fq_batched_swiglu_quant_bwd(*s["args"]))
+                _lib.check(bwd_fn(*s["args"]))
 
             def cpu_fn():
                 from oracle import fq_oracle as O
@@ -234,21 +250,29 @@ def build_cases(names, dev):
             nbytes = configs.rw_batched_swiglu_bwd(M, n, counts)
             entry = "triton_batch_weighted_silu_and_block_quant_backward"
         else:
+            fwd_fn = L.fq_batched_swiglu_quant_fwd_planned if planned else L.fq_batched_swiglu_quant_fwd
+
             def launch(s):
-                _lib.check(L.fq_batched_swiglu_quant_fwd(*s["args"]))
+                _lib.check(fwd_fn(*s["args"]))
 
             def cpu_fn():
                 from oracle import fq_oracle as O
                 return O.batch_weighted_silu_and_block_quant_forward(x_cpu, w_cpu, counts, False)
             nbytes = configs.rw_batched_swiglu_fwd(M, n, counts)
             entry = "triton_batch_weighted_silu_and_block_quant_forward(output_mode=2)"
-        c = Case("cfg3b" if backward else "cfg3", entry, [M, N], nbytes, make_set, launch, cpu_fn)
+        if planned:
+            entry += " with plan="
+        c = Case(("cfg3b" if backward else "cfg3") + ("_planned" if planned else ""), entry, [M, N], nbytes,
+                 make_set, launch, cpu_fn)
         c.extra = dict(n_experts=E, blocks=blocks, empty_experts=sum(1 for v in counts if v == 0),
                        max_count=max(counts))
         return c
 
     add("cfg3", build=lambda: batched_case(False))
     add("cfg3b", build=lambda: batched_case(True))
+    # the same with every workgroup's tile read from a plan built once from the counts
+    add("cfg3_planned", build=lambda: batched_case(False, True))
+    add("cfg3b_planned", build=lambda: batched_case(True, True))
 
     # ---------------------------------------------------------------- cfg4
     def swiglu_bwd_case(kind, name, pow2=False):
@@ -404,6 +428,9 @@ def build_cases(names, dev):
     # ---------------------------------------------------------------- the quantisers with no fused pre-op
     def plain_quant_case(name):
         g = torch.Generator().manual_seed(1105)
+        planned = name == "a8_batch_blockwise_planned"
+        if planned:
+            name = "a8_batch_blockwise"
         if name == "a8_batch_blockwise":  # the activations of cfg3's experts: 65536 x 512, same Zipf counts
             d = lazy.setdefault("cfg3", configs.cfg3_batched_swiglu())
             counts = d["counts"]
@@ -414,6 +441,7 @@ def build_cases(names, dev):
         x_cpu = torch.randn(M, N, generator=g).to(torch.bfloat16)
         blocks = sum((c + 127) // 128 for c in counts) if counts else (M + 127) // 128
         cnt = torch.tensor(counts, dtype=torch.int32, device=dev) if counts else None
+        plan, pshape = expert_plan(cnt, counts) if planned else (None, None)
 
         def make_set():
             s = dict(x=x_cpu.to(dev), q=torch.empty((M, N), device=dev, dtype=FP8),
@@ -426,13 +454,17 @@ def build_cases(names, dev):
                              stream)
             elif name == "a8_group":
                 s["args"] = (_p(s["x"]), _p(s["q"]), _p(s["s"]), M, N, 0, _lib.FQ_E4M3, stream)
+            elif planned:
+                s["args"] = (_p(s["x"]), _p(plan), pshape, _p(s["q"]), _p(s["s"]), _p(s["qt"]), _p(s["st"]), M, N, 0,
+                             _lib.FQ_E4M3, stream)
             else:
                 s["args"] = (_p(s["x"]), _p(cnt), 0, len(counts), blocks, _p(s["q"]), _p(s["s"]), _p(s["qt"]),
                              _p(s["st"]), M, N, 0, _lib.FQ_E4M3, stream)
             return s
 
         fn = {"a8_blockwise": L.fq_blockwise_quant, "a8_group": L.fq_group_quant,
-              "a8_batch_blockwise": L.fq_batched_blockwise_quant}[name]
+              "a8_batch_blockwise": L.fq_batched_blockwise_quant_planned if planned
+              else L.fq_batched_blockwise_quant}[name]
 
         def launch(s):
             _lib.check(fn(*s["args"]))
@@ -449,10 +481,11 @@ def build_cases(names, dev):
         col = M * N + 4 * blocks * N
         entry = {"a8_blockwise": "triton_blockwise_quant(output_mode=2)", "a8_group": "triton_group_quant",
                  "a8_batch_blockwise": "triton_batch_blockwise_quant"}[name]
-        return Case(name, entry, [M, N], (2 * M * N, row + (0 if name == "a8_group" else col)), make_set, launch,
-                    cpu_fn)
+        c = Case(name + ("_planned" if planned else ""), entry + (" with plan=" if planned else ""), [M, N],
+                 (2 * M * N, row + (0 if name == "a8_group" else col)), make_set, launch, cpu_fn)
+        return c
 
-    for _n in ("a8_blockwise", "a8_group", "a8_batch_blockwise"):
+    for _n in ("a8_blockwise", "a8_group", "a8_batch_blockwise", "a8_batch_blockwise_planned"):
         add(_n, build=lambda _n=_n: plain_quant_case(_n))
 
     # ---------------------------------------------------------------- next row: RMSNorm + router GEMM + quant
@@ -744,6 +777,7 @@ def load_traffic_table():
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
        "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg5b_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
+       "cfg3_planned", "cfg3b_planned", "a8_batch_blockwise_planned",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed", "next_router_wide",
        "stream_read", "stream_copy"]
 

@@ -83,6 +83,35 @@ int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_
                                int64_t total_blocks, void* q, float* s, void* qt, float* st, int64_t M,
                                int64_t N, int round_scale, int fp8_kind, void* stream);
 
+/* The per-expert entry points find every workgroup's tile by a prefix scan over
+ * the device-side counts.  A caller that runs several of them on the same
+ * counts (the forward, the backward and the quantiser of one MoE layer) can
+ * have that scan done once, and the launches sized for exactly the workgroups
+ * that have a tile:
+ *  - fq_expert_plan_shape (host only, no GPU work) reads the caller's host-side
+ *    copy of the counts - what the reference takes as `splits`
+ *    (linghe/utils/silu.py:826, :838: "batch mode need splits to launch
+ *    kernels") - and fills shape[0..3]: the number of 128-row blocks
+ *    (= total_blocks of the other forms) and how many of them are worked on
+ *    whole, in halves and in quarters;
+ *  - fq_build_expert_plan writes one 16-byte record per row block from the
+ *    DEVICE-side counts into `plan` (fq_expert_plan_bytes(shape) bytes of
+ *    device memory, 16-byte aligned);
+ *  - the *_planned forms of the entry points take plan and shape in place of
+ *    counts, n_experts and total_blocks.  Their outputs are identical to those
+ *    of the forms that take the counts.  A plan addresses at most 2^31 - 1 rows.
+ * Where host and device counts disagree the row blocks concerned are left out,
+ * as in the other forms. */
+int fq_expert_plan_shape(const int64_t* host_counts, int n_experts, int64_t* shape);
+int64_t fq_expert_plan_bytes(const int64_t* shape);
+int fq_build_expert_plan(const void* counts, int counts_is_i64, int n_experts, const int64_t* shape, void* plan,
+                         void* stream);
+
+/* fq_batched_blockwise_quant with the tiles read from a plan. */
+int fq_batched_blockwise_quant_planned(const void* x, const void* plan, const int64_t* shape, void* q, float* s,
+                                       void* qt, float* st, int64_t M, int64_t N, int round_scale, int fp8_kind,
+                                       void* stream);
+
 /* triton_batch_block_pad_permute_with_indices, linghe/utils/gather.py:960-1113
  * (kernel :840-957).  x bf16 [src_rows, N]; indices int32 [M], M = sum of the
  * counts each rounded up to 16: expert e's region of the outputs starts at the
@@ -214,6 +243,16 @@ int fq_batched_swiglu_quant_bwd(const void* g, const void* x, const void* weight
                                 const void* counts, int counts_is_i64, int n_experts, int64_t total_blocks,
                                 void* dq, float* ds, void* dw, void* dqt, float* dst, float* dw_partials,
                                 int64_t M, int64_t n, int round_scale, int fp8_kind, void* stream);
+
+/* The two entry points above with the tiles read from a plan
+ * (fq_build_expert_plan). */
+int fq_batched_swiglu_quant_fwd_planned(const void* x, const void* weight, int weight_is_bf16, const void* plan,
+                                        const int64_t* shape, void* q, float* s, void* qt, float* st, int64_t M,
+                                        int64_t n, int round_scale, int output_mode, int fp8_kind, void* stream);
+int fq_batched_swiglu_quant_bwd_planned(const void* g, const void* x, const void* weight, int weight_is_bf16,
+                                        const void* plan, const int64_t* shape, void* dq, float* ds, void* dw,
+                                        void* dqt, float* dst, float* dw_partials, int64_t M, int64_t n,
+                                        int round_scale, int fp8_kind, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,6 +30,9 @@ SIGNATURES = {
     "fq_stream_rw_variant": [_P, _L, _P, _L, _P, _I, _L, _I, _I, _I, _P],
     "fq_blockwise_quant": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_blockwise_quant": [_P, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _P],
+    "fq_batched_blockwise_quant_planned": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
+    "fq_expert_plan_shape": [_P, _I, _P],
+    "fq_build_expert_plan": [_P, _I, _I, _P, _P, _P],
     "fq_batched_pad_permute_quant": [_P, _P, _I, _I, _L, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _P],
     "fq_block_quant": [_P, _P, _P, _L, _L, _I, _I, _P],
     "fq_swiglu_fwd": [_P, _P, _I, _P, _L, _L, _P],
@@ -46,8 +49,11 @@ SIGNATURES = {
     "fq_swiglu_quant_bwd": [_P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_swiglu_quant_fwd": [_P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_swiglu_quant_bwd": [_P, _P, _P, _I, _P, _I, _I, _L, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
+    "fq_batched_swiglu_quant_fwd_planned": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
+    "fq_batched_swiglu_quant_bwd_planned": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
 }
-OTHER_SYMBOLS = ["fq_version", "fq_last_error", "fq_rmsnorm_bwd_num_partials", "fq_rmsnorm_router_scratch_bytes"]
+OTHER_SYMBOLS = ["fq_version", "fq_last_error", "fq_rmsnorm_bwd_num_partials", "fq_rmsnorm_router_scratch_bytes",
+                 "fq_expert_plan_bytes"]
 
 
 def _load() -> ctypes.CDLL:
@@ -68,6 +74,8 @@ def _load() -> ctypes.CDLL:
     lib.fq_rmsnorm_bwd_num_partials.restype = _L
     lib.fq_rmsnorm_router_scratch_bytes.argtypes = [_L, _L, _I]
     lib.fq_rmsnorm_router_scratch_bytes.restype = _L
+    lib.fq_expert_plan_bytes.argtypes = [_P]
+    lib.fq_expert_plan_bytes.restype = _L
     return lib
 
 

@@ -103,20 +103,104 @@ int fq_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, in
                       fn);
 }
 
-int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
-                               int64_t total_blocks, void* q, float* s, void* qt, float* st, int64_t M,
-                               int64_t N, int round_scale, int fp8_kind, void* stream) {
-  const char* fn = "fq_batched_blockwise_quant";
+}  // extern "C"
+
+// The per-expert entry points come in two forms that differ only in where a workgroup learns its
+// tile: from the device-side counts, or from a plan built from them (counts NULL, n_experts unused).
+static int check_plan_shape(const char* fn, const int64_t* shape, fq::PlanShape* ps) {
+  FQ_REQUIRE(shape != nullptr, FQ_ERR_ARG, "%s: plan shape NULL", fn);
+  FQ_REQUIRE(shape[1] >= 0 && shape[2] >= 0 && shape[3] >= 0 && shape[0] == shape[1] + shape[2] + shape[3] &&
+                 shape[0] <= (int64_t)0x3fffffff,
+             FQ_ERR_SHAPE, "%s: not a plan shape (fq_expert_plan_shape fills it)", fn);
+  ps->unpacked = shape[1];
+  ps->packed2 = shape[2];
+  ps->packed4 = shape[3];
+  return FQ_OK;
+}
+
+static int check_batch_source(const char* fn, const void* counts, int n_experts, const void* plan,
+                              int64_t total_blocks, int64_t M) {
+  FQ_REQUIRE(total_blocks >= 0, FQ_ERR_SHAPE, "%s: negative block count", fn);
+  if (plan != nullptr) {
+    FQ_REQUIRE(aligned16(plan), FQ_ERR_ARG, "%s: plan misaligned", fn);
+    // every row block holds at least one row
+    FQ_REQUIRE(total_blocks <= M, FQ_ERR_SHAPE, "%s: plan shape inconsistent with M", fn);
+    FQ_REQUIRE(M <= (int64_t)0x7fffffff, FQ_ERR_SHAPE, "%s: a plan addresses at most 2^31 - 1 rows", fn);
+    return FQ_OK;
+  }
+  FQ_REQUIRE(n_experts >= 0, FQ_ERR_SHAPE, "%s: negative expert count", fn);
+  FQ_REQUIRE(counts != nullptr, FQ_ERR_ARG, "%s: counts NULL", fn);
+  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
+  return FQ_OK;
+}
+
+static int batched_blockwise_quant(const char* fn, const void* x, const void* counts, int counts_is_i64,
+                                   int n_experts, const void* plan, const fq::PlanShape* ps, int64_t total_blocks,
+                                   void* q, float* s, void* qt, float* st, int64_t M, int64_t N, int round_scale,
+                                   int fp8_kind, void* stream) {
   int rc = check_common(fn, M, N, round_scale, fp8_kind);
   if (rc) return rc;
   if ((rc = check_mode_ptrs(fn, 2, q, s, qt, st))) return rc;
-  FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0, FQ_ERR_SHAPE, "%s: negative expert/block count", fn);
+  FQ_REQUIRE((plan != nullptr || n_experts >= 0) && total_blocks >= 0, FQ_ERR_SHAPE,
+             "%s: negative expert/block count", fn);
   if (M == 0 || total_blocks == 0) return FQ_OK;
-  FQ_REQUIRE(x && aligned16(x) && counts, FQ_ERR_ARG, "%s: x/counts NULL or x misaligned", fn);
-  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
+  FQ_REQUIRE(x && aligned16(x), FQ_ERR_ARG, "%s: x NULL or misaligned", fn);
+  if ((rc = check_batch_source(fn, counts, n_experts, plan, total_blocks, M))) return rc;
   if ((rc = check_tiles(fn, total_blocks * (N / 128)))) return rc;
   return check_launch(fq::launch_blockwise_quant(x, q, s, qt, st, M, (int)N, round_scale, 2, fp8_kind, counts,
-                                                 counts_is_i64 != 0, n_experts, total_blocks, (hipStream_t)stream),
+                                                 counts_is_i64 != 0, n_experts, total_blocks, (hipStream_t)stream,
+                                                 plan, ps),
+                      fn);
+}
+
+extern "C" {
+
+int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
+                               int64_t total_blocks, void* q, float* s, void* qt, float* st, int64_t M,
+                               int64_t N, int round_scale, int fp8_kind, void* stream) {
+  return batched_blockwise_quant("fq_batched_blockwise_quant", x, counts, counts_is_i64, n_experts, nullptr, nullptr,
+                                 total_blocks, q, s, qt, st, M, N, round_scale, fp8_kind, stream);
+}
+
+int fq_batched_blockwise_quant_planned(const void* x, const void* plan, const int64_t* shape, void* q, float* s,
+                                       void* qt, float* st, int64_t M, int64_t N, int round_scale, int fp8_kind,
+                                       void* stream) {
+  const char* fn = "fq_batched_blockwise_quant_planned";
+  fq::PlanShape ps;
+  int rc = check_plan_shape(fn, shape, &ps);
+  if (rc) return rc;
+  FQ_REQUIRE(plan != nullptr || M == 0 || shape[0] == 0, FQ_ERR_ARG, "%s: plan NULL", fn);
+  return batched_blockwise_quant(fn, x, nullptr, 0, 0, plan, &ps, shape[0], q, s, qt, st, M, N, round_scale, fp8_kind,
+                                 stream);
+}
+
+int fq_expert_plan_shape(const int64_t* host_counts, int n_experts, int64_t* shape) {
+  const char* fn = "fq_expert_plan_shape";
+  FQ_REQUIRE(n_experts >= 0 && shape != nullptr && (host_counts != nullptr || n_experts == 0), FQ_ERR_ARG,
+             "%s: NULL pointer or negative expert count", fn);
+  const fq::PlanShape ps = fq::expert_plan_shape(host_counts, n_experts);
+  FQ_REQUIRE(ps.blocks() <= (int64_t)0x3fffffff, FQ_ERR_SHAPE, "%s: more than 2^30 - 1 row blocks", fn);
+  shape[0] = ps.blocks();
+  shape[1] = ps.unpacked;
+  shape[2] = ps.packed2;
+  shape[3] = ps.packed4;
+  return FQ_OK;
+}
+
+int64_t fq_expert_plan_bytes(const int64_t* shape) {
+  return shape == nullptr || shape[0] < 0 ? 0 : shape[0] * 16;
+}
+
+int fq_build_expert_plan(const void* counts, int counts_is_i64, int n_experts, const int64_t* shape, void* plan,
+                         void* stream) {
+  const char* fn = "fq_build_expert_plan";
+  fq::PlanShape ps;
+  int rc = check_plan_shape(fn, shape, &ps);
+  if (rc) return rc;
+  FQ_REQUIRE(n_experts >= 0, FQ_ERR_SHAPE, "%s: negative expert count", fn);
+  if (shape[0] == 0) return FQ_OK;
+  FQ_REQUIRE(plan && aligned16(plan) && (counts || n_experts == 0), FQ_ERR_ARG, "%s: NULL or misaligned pointer", fn);
+  return check_launch(fq::launch_expert_plan(counts, counts_is_i64 != 0, n_experts, ps, plan, (hipStream_t)stream),
                       fn);
 }
 
@@ -379,43 +463,92 @@ int fq_swiglu_quant_bwd(const void* g, const void* x, void* dq, float* ds, void*
                       fn);
 }
 
+}  // extern "C"
+
+static int batched_swiglu_quant_fwd(const char* fn, const void* x, const void* weight, int weight_is_bf16,
+                                    const void* counts, int counts_is_i64, int n_experts, const void* plan,
+                                    const fq::PlanShape* ps, int64_t total_blocks, void* q, float* s, void* qt,
+                                    float* st, int64_t M, int64_t n, int round_scale, int output_mode,
+                                    int fp8_kind, void* stream) {
+  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, output_mode, q, s, qt, st))) return rc;
+  FQ_REQUIRE((plan != nullptr || n_experts >= 0) && total_blocks >= 0, FQ_ERR_SHAPE,
+             "%s: negative expert/block count", fn);
+  if (M == 0 || total_blocks == 0) return FQ_OK;
+  FQ_REQUIRE(x && aligned16(x) && weight, FQ_ERR_ARG, "%s: NULL or misaligned input", fn);
+  if ((rc = check_batch_source(fn, counts, n_experts, plan, total_blocks, M))) return rc;
+  if ((rc = check_tiles(fn, total_blocks * (n / 128)))) return rc;
+  return check_launch(fq::launch_silu_quant_fwd(x, weight, weight_is_bf16 != 0, q, s, qt, st, M, (int)n, round_scale,
+                                                output_mode, fp8_kind, counts, counts_is_i64 != 0, n_experts,
+                                                total_blocks, (hipStream_t)stream, plan, ps),
+                      fn);
+}
+
+static int batched_swiglu_quant_bwd(const char* fn, const void* g, const void* x, const void* weight,
+                                    int weight_is_bf16, const void* counts, int counts_is_i64, int n_experts,
+                                    const void* plan, const fq::PlanShape* ps, int64_t total_blocks, void* dq,
+                                    float* ds, void* dw, void* dqt, float* dst, float* dw_partials, int64_t M,
+                                    int64_t n, int round_scale, int fp8_kind, void* stream) {
+  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  if (rc) return rc;
+  if ((rc = check_mode_ptrs(fn, 2, dq, ds, dqt, dst))) return rc;
+  FQ_REQUIRE((plan != nullptr || n_experts >= 0) && total_blocks >= 0, FQ_ERR_SHAPE,
+             "%s: negative expert/block count", fn);
+  if (M == 0 || total_blocks == 0) return FQ_OK;
+  FQ_REQUIRE(g && x && aligned16(g) && aligned16(x) && weight && dw && dw_partials, FQ_ERR_ARG,
+             "%s: NULL or misaligned pointer", fn);
+  if ((rc = check_batch_source(fn, counts, n_experts, plan, total_blocks, M))) return rc;
+  if ((rc = check_tiles(fn, total_blocks * (n / 128)))) return rc;
+  return check_launch(fq::launch_silu_quant_bwd(g, x, weight, weight_is_bf16 != 0, dq, ds, dqt, dst, dw_partials, dw,
+                                                M, (int)n, round_scale, fp8_kind, counts, counts_is_i64 != 0,
+                                                n_experts, total_blocks, (hipStream_t)stream, plan, ps),
+                      fn);
+}
+
+extern "C" {
+
 int fq_batched_swiglu_quant_fwd(const void* x, const void* weight, int weight_is_bf16, const void* counts,
                                 int counts_is_i64, int n_experts, int64_t total_blocks, void* q, float* s,
                                 void* qt, float* st, int64_t M, int64_t n, int round_scale, int output_mode,
                                 int fp8_kind, void* stream) {
-  const char* fn = "fq_batched_swiglu_quant_fwd";
-  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  return batched_swiglu_quant_fwd("fq_batched_swiglu_quant_fwd", x, weight, weight_is_bf16, counts, counts_is_i64,
+                                  n_experts, nullptr, nullptr, total_blocks, q, s, qt, st, M, n, round_scale,
+                                  output_mode, fp8_kind, stream);
+}
+
+int fq_batched_swiglu_quant_fwd_planned(const void* x, const void* weight, int weight_is_bf16, const void* plan,
+                                        const int64_t* shape, void* q, float* s, void* qt, float* st, int64_t M,
+                                        int64_t n, int round_scale, int output_mode, int fp8_kind, void* stream) {
+  const char* fn = "fq_batched_swiglu_quant_fwd_planned";
+  fq::PlanShape ps;
+  int rc = check_plan_shape(fn, shape, &ps);
   if (rc) return rc;
-  if ((rc = check_mode_ptrs(fn, output_mode, q, s, qt, st))) return rc;
-  FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0, FQ_ERR_SHAPE, "%s: negative expert/block count", fn);
-  if (M == 0 || total_blocks == 0) return FQ_OK;
-  FQ_REQUIRE(x && aligned16(x) && weight && counts, FQ_ERR_ARG, "%s: NULL or misaligned input", fn);
-  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
-  if ((rc = check_tiles(fn, total_blocks * (n / 128)))) return rc;
-  return check_launch(fq::launch_silu_quant_fwd(x, weight, weight_is_bf16 != 0, q, s, qt, st, M, (int)n, round_scale,
-                                                output_mode, fp8_kind, counts, counts_is_i64 != 0, n_experts,
-                                                total_blocks, (hipStream_t)stream),
-                      fn);
+  FQ_REQUIRE(plan != nullptr || M == 0 || shape[0] == 0, FQ_ERR_ARG, "%s: plan NULL", fn);
+  return batched_swiglu_quant_fwd(fn, x, weight, weight_is_bf16, nullptr, 0, 0, plan, &ps, shape[0], q, s, qt, st, M,
+                                  n, round_scale, output_mode, fp8_kind, stream);
 }
 
 int fq_batched_swiglu_quant_bwd(const void* g, const void* x, const void* weight, int weight_is_bf16,
                                 const void* counts, int counts_is_i64, int n_experts, int64_t total_blocks,
                                 void* dq, float* ds, void* dw, void* dqt, float* dst, float* dw_partials,
                                 int64_t M, int64_t n, int round_scale, int fp8_kind, void* stream) {
-  const char* fn = "fq_batched_swiglu_quant_bwd";
-  int rc = check_common(fn, M, n, round_scale, fp8_kind);
+  return batched_swiglu_quant_bwd("fq_batched_swiglu_quant_bwd", g, x, weight, weight_is_bf16, counts, counts_is_i64,
+                                  n_experts, nullptr, nullptr, total_blocks, dq, ds, dw, dqt, dst, dw_partials, M, n,
+                                  round_scale, fp8_kind, stream);
+}
+
+int fq_batched_swiglu_quant_bwd_planned(const void* g, const void* x, const void* weight, int weight_is_bf16,
+                                        const void* plan, const int64_t* shape, void* dq, float* ds, void* dw,
+                                        void* dqt, float* dst, float* dw_partials, int64_t M, int64_t n,
+                                        int round_scale, int fp8_kind, void* stream) {
+  const char* fn = "fq_batched_swiglu_quant_bwd_planned";
+  fq::PlanShape ps;
+  int rc = check_plan_shape(fn, shape, &ps);
   if (rc) return rc;
-  if ((rc = check_mode_ptrs(fn, 2, dq, ds, dqt, dst))) return rc;
-  FQ_REQUIRE(n_experts >= 0 && total_blocks >= 0, FQ_ERR_SHAPE, "%s: negative expert/block count", fn);
-  if (M == 0 || total_blocks == 0) return FQ_OK;
-  FQ_REQUIRE(g && x && aligned16(g) && aligned16(x) && weight && counts && dw && dw_partials, FQ_ERR_ARG,
-             "%s: NULL or misaligned pointer", fn);
-  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
-  if ((rc = check_tiles(fn, total_blocks * (n / 128)))) return rc;
-  return check_launch(fq::launch_silu_quant_bwd(g, x, weight, weight_is_bf16 != 0, dq, ds, dqt, dst, dw_partials, dw,
-                                                M, (int)n, round_scale, fp8_kind, counts, counts_is_i64 != 0,
-                                                n_experts, total_blocks, (hipStream_t)stream),
-                      fn);
+  FQ_REQUIRE(plan != nullptr || M == 0 || shape[0] == 0, FQ_ERR_ARG, "%s: plan NULL", fn);
+  return batched_swiglu_quant_bwd(fn, g, x, weight, weight_is_bf16, nullptr, 0, 0, plan, &ps, shape[0], dq, ds, dw, dqt,
+                                  dst, dw_partials, M, n, round_scale, fp8_kind, stream);
 }
 
 }  // extern "C"

@@ -7,9 +7,17 @@
 
 namespace fq {
 
+// Sizes of the three sections of a per-expert tile plan: row blocks worked on unpacked, last blocks
+// of 33..64 rows, last blocks of at most 32 rows (counted on the host from its copy of the counts)
+struct PlanShape {
+  int64_t unpacked, packed2, packed4;
+  int64_t blocks() const { return unpacked + packed2 + packed4; }
+};
+
 hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int N,
                                   int round_scale, int mode, int kind, const void* counts, int counts_i64,
-                                  int n_experts, int64_t row_blocks, hipStream_t stream);
+                                  int n_experts, int64_t row_blocks, hipStream_t stream, const void* plan = nullptr,
+                                  const PlanShape* ps = nullptr);
 
 hipError_t launch_pad_permute_quant(const void* x, const void* indices, const void* probs, int probs_bf16,
                                     void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
@@ -19,12 +27,21 @@ hipError_t launch_pad_permute_quant(const void* x, const void* indices, const vo
 hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_bf16, void* q, float* s, void* qt,
                                  float* st, int64_t M, int n, int round_scale, int mode, int kind,
                                  const void* counts, int counts_i64, int n_experts, int64_t row_blocks,
-                                 hipStream_t stream);
+                                 hipStream_t stream, const void* plan = nullptr, const PlanShape* ps = nullptr);
 
 hipError_t launch_silu_quant_bwd(const void* g, const void* x, const void* weight, int weight_bf16, void* q,
                                  float* s, void* qt, float* st, float* dw_part, void* dw, int64_t M, int n,
                                  int round_scale, int kind, const void* counts, int counts_i64, int n_experts,
-                                 int64_t row_blocks, hipStream_t stream);
+                                 int64_t row_blocks, hipStream_t stream, const void* plan = nullptr,
+                                  const PlanShape* ps = nullptr);
+
+// Per-expert launches with `plan` (expert_plan_bytes(ps) bytes of device memory filled by
+// launch_expert_plan from the same counts) and its shape read their tile from it instead of
+// scanning the counts; counts may then be NULL and row_blocks is not used.
+PlanShape expert_plan_shape(const int64_t* host_counts, int n_experts);
+int64_t expert_plan_bytes(const PlanShape& ps);
+hipError_t launch_expert_plan(const void* counts, int counts_i64, int n_experts, const PlanShape& ps, void* plan,
+                              hipStream_t stream);
 
 hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const float* rstd, void* q, float* s,
                                      void* qt, float* st, int64_t M, int n, int round_scale, int mode, int kind,

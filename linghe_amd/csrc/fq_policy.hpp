@@ -72,6 +72,12 @@ struct Policy {
   // waves (one row each) per workgroup of the statistic pass: 18.10 / 18.00 / 18.00 / 18.04 us at 8192 x 2048 and
   // 107.8 / 108.0 / 107.4 / 107.6 at 16384 x 7168 with 1 / 2 / 4 / 8
   static constexpr int kRowstatWaves = 4;
+  // per-expert launches that read their tiles from a plan: the packed tiles (last row blocks of at most 64
+  // rows) before or behind the others.  65536 rows in 256 experts (Zipf counts), packed first / last:
+  // SwiGLU forward 44.2 / 43.2 us, backward 77.7 / 77.4, blockwise quantiser 30.9 / 31.8
+  static constexpr bool kPlanPackedFirstSiluFwd = false;
+  static constexpr bool kPlanPackedFirstSiluBwd = false;
+  static constexpr bool kPlanPackedFirstBlockwise = true;
   static constexpr bool kStartPriorityRmsnorm = true;
   // 16-byte chunks per lane, matrix and step in the bf16 SwiGLU backward (three matrices are read):
   // 29.0 / 30.4 / 28.7 / 35.5 us with 2 / 3 / 4 / 8 at 8192 x 4096

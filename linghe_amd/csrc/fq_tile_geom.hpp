@@ -27,7 +27,38 @@ struct BatchArgs {
   int counts_i64;
   int n_experts;
   int pad;             // 0/1: experts packed back to back; 16: each expert's region padded to 16 rows
+  const void* plan;    // device, PlanEntry per 128-row block (expert_plan_kernel), or NULL: scan the counts
+  int plan_unpacked;   // records of row blocks that are worked on unpacked,
+  int plan_packed2;    // of last blocks of 33..64 rows, and (behind them) of
+  int plan_packed4;    // last blocks of at most 32 rows: the table's three sections, counted by the host
+  int plan_packed_first;  // order of a planned launch: the packed tiles before (1) or behind (0) the others
 };
+
+// What a workgroup of a per-expert launch needs to know about its 128-row block, written once per
+// set of counts by expert_plan_kernel and read with one 16-byte load through the constant path
+// instead of the prefix scan over all counts (which puts a dependent vector load and three wave
+// scans in front of every workgroup's first tile load).  Experts lie back to back (no padding of
+// their regions).  Three sections, each in expert order: the row blocks that are worked on
+// unpacked (all but an expert's last one, and last ones of more than 64 rows), the last blocks of
+// 33..64 rows (two column blocks to a workgroup), the last blocks of at most 32 rows (four).  The
+// host knows the sizes of the sections from its copy of the counts, sizes the launch for exactly
+// the workgroups that have a tile, and passes the sizes as kernel arguments: a workgroup finds its
+// section and its record from its number alone.
+// Records are small because they are read cold: every line of the table that a workgroup is the
+// first of its XCD to touch costs it a trip to memory before its first tile load can leave.
+struct PlanEntry {
+  uint32_t row0;   // first global row of the row block
+  int rb;          // row block inside the expert
+  int count;       // rows of the expert
+  uint32_t where;  // kind << 30 | row block in expert order over all experts (row of the transposed scales)
+};
+constexpr uint32_t kPlanEmpty = 0, kPlanUnpacked = 1, kPlanPacked2 = 2, kPlanPacked4 = 3;  // kinds
+static_assert(sizeof(PlanEntry) == 16, "16-byte records");
+
+// workgroups of a planned launch over ncb column blocks
+__host__ __device__ inline int64_t plan_workgroups(int64_t unpacked, int64_t packed2, int64_t packed4, int ncb) {
+  return unpacked * ncb + packed2 * ((ncb + 1) >> 1) + packed4 * ((ncb + 3) >> 2);
+}
 
 // out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
 // backward's dx1|dx2)
@@ -66,6 +97,56 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
     g.st_row = rbk;
     g.expert = 0;
     g.valid = left > 0;
+  } else if (b.plan != nullptr) {  // workgroup-uniform
+    typedef const __attribute__((address_space(4))) uint32_t* const_u32;
+    const int c1 = (ncb + 1) >> 1, c2 = (ncb + 3) >> 2;
+    // Order of the launch: the packed tiles, which move few bytes for the time they take, before or
+    // behind the unpacked row blocks (those in expert order: neighbouring row blocks of an expert
+    // share lines of the transposed outputs, and a strided walk over them measured 20 % slower).
+    // Which end is better differs by kernel, by about 1 us either way at 65536 rows in 256 experts.
+    const int n1 = b.plan_packed2 * c1, n2 = b.plan_packed4 * c2;
+    int idx, x;
+    uint32_t kind = kPlanUnpacked;
+    if (!b.plan_packed_first) {
+      const int n0 = b.plan_unpacked * ncb;
+      id = id < n0 ? id + n1 + n2 : id - n0;
+    }
+    if (id < n1) {
+      const int q = id / c1;
+      idx = b.plan_unpacked + q;
+      x = id - q * c1;
+      kind = kPlanPacked2;
+    } else if (id < n1 + n2) {
+      const int r = id - n1, q = r / c2;
+      idx = b.plan_unpacked + b.plan_packed2 + q;
+      x = r - q * c2;
+      kind = kPlanPacked4;
+    } else {
+      const int r = id - n1 - n2;
+      idx = r / ncb;
+      x = r - idx * ncb;
+    }
+    const_u32 e = (const_u32)((uintptr_t)b.plan + (uintptr_t)idx * sizeof(PlanEntry));
+    const uint32_t row0 = e[0], where = e[3];
+    const int rb = (int)e[1], count = (int)e[2];
+    g.kc_shift = (int)kind - 1;
+    const int64_t row_start = (int64_t)row0 - (int64_t)rb * kGroup;
+    const int left = count - rb * kGroup;
+    g.cb = x << g.kc_shift;
+    const int cbs_left = ncb - g.cb;
+    g.n_sub = cbs_left < (1 << g.kc_shift) ? cbs_left : (1 << g.kc_shift);
+    // a record of another kind than its section's: the host's counts are not the device's
+    g.valid = (where >> 30) == kind && idx < b.plan_unpacked + b.plan_packed2 + b.plan_packed4;
+    g.expert = 0;  // not recorded: no kernel that takes a plan asks for it
+    g.rows_valid = left < kGroup ? left : kGroup;
+    g.rows_store = g.rows_valid;
+    g.row0 = (int64_t)row0;
+    g.s_base = row_start * (out_w / kGroup) + (int64_t)rb * kGroup;
+    g.s_stride = count;
+    g.t_base = row_start * out_w + (int64_t)rb * kGroup;
+    g.t_stride = count;
+    g.st_row = (int64_t)(where & 0x3fffffffu);
+    if (g.row0 + g.rows_store > M) g.valid = false;
   } else {
     const ExpertTile et = find_expert_tile(b.counts, b.counts_i64, b.n_experts, id, ncb, b.pad > 1 ? b.pad : 1);
     // the lookup's answer is the same in every lane: keep it in scalar registers

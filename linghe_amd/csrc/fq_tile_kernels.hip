@@ -305,7 +305,7 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadRmsnorm) void rmsnorm_
   // lets the newcomers push aside the stores of the ones at work: 4 % slower at 16384 x 7168.
   if (first) __builtin_amdgcn_s_setprio(3);
   __shared__ TileShared<RPT> sh;
-  BatchArgs none{nullptr, 0, 0};
+  BatchArgs none{nullptr, 0, 0, 0, nullptr, 0, 0, 0, 0};
   const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none, remap);
   if (!g.valid) return;
   uint4 raw[RPT];
@@ -336,16 +336,146 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadRmsnorm) void rmsnorm_
 }
 
 // ---------------------------------------------------------------------------
+// The per-row-block table of a set of counts (PlanEntry): one workgroup of 1024 threads, one
+// expert per thread and pass.  Every pass scans its experts' row blocks, rows and the members of
+// the table's three sections over the workgroup, leaves the exclusive sums in shared memory and
+// writes the pass's records, one per thread and step, each finding its expert by bisection over
+// the exclusive block sums.  The sizes of the sections are the host's; where the device-side
+// counts give a section fewer members the rest of it is marked empty, where they give it more the
+// surplus is dropped (the launches then leave those row blocks out: the counts disagree).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restrict__ counts, int counts_i64,
+                                                           int n_experts, int b0, int b1, int b2,
+                                                           PlanEntry* __restrict__ plan) {
+  constexpr int T = 1024, W = T / 64;
+  __shared__ int eb[T + 1];  // exclusive sums of the pass: row blocks,
+  __shared__ int ez[T];      // unpacked row blocks,
+  __shared__ int ep[T];      // packed last blocks (two-fold in the low half, four-fold in the high half),
+  __shared__ int64_t er[T];  // rows
+  __shared__ int ec[T];      // the counts themselves
+  __shared__ int wb[W], wz[W], wp[W];
+  __shared__ int64_t wr[W];
+  __shared__ int pass_z, pass_p;
+  const int t = (int)tid_x(), lane = t & 63, wave = t >> 6;
+  int64_t run_rows = 0;
+  int run_blocks = 0, run_z = 0, run_p1 = 0, run_p2 = 0;
+  for (int base = 0; base < n_experts; base += T) {
+    const int e = base + t;
+    const int cr = e < n_experts ? load_count(counts, counts_i64, e) : 0;
+    const int c = cr > 0 ? cr : 0;
+    const int nb = (c + kGroup - 1) / kGroup;
+    const int sh = nb > 0 ? pack_shift(c - (nb - 1) * kGroup) : 0;
+    const int p = (sh == 1) + ((sh == 2) << 16);
+    const int z = nb - (sh > 0);
+    const int ib = wave_inclusive_scan(nb);
+    const int iz = wave_inclusive_scan(z);
+    const int ip = wave_inclusive_scan(p);
+    // the rows of 64 experts fit 32 bits for every matrix the entry points accept; the sums over
+    // waves and passes are 64-bit
+    const int ir = wave_inclusive_scan(c);
+    if (lane == 63) { wb[wave] = ib; wz[wave] = iz; wp[wave] = ip; wr[wave] = ir; }
+    __syncthreads();
+    int ob = 0, oz = 0, op = 0;
+    int64_t orow = 0;
+    for (int w = 0; w < wave; ++w) { ob += wb[w]; oz += wz[w]; op += wp[w]; orow += wr[w]; }
+    eb[t] = ob + ib - nb;
+    ez[t] = oz + iz - z;
+    ep[t] = op + ip - p;
+    er[t] = orow + ir - c;
+    ec[t] = c;
+    if (t == T - 1) {
+      eb[T] = ob + ib;
+      pass_z = oz + iz;
+      pass_p = op + ip;
+    }
+    __syncthreads();
+    const int pass_blocks = eb[T];
+    for (int j = t; j < pass_blocks; j += T) {
+      int lo = 0, hi = T - 1;  // the last expert of the pass whose exclusive sum is <= j
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (eb[mid] <= j) lo = mid; else hi = mid - 1;
+      }
+      const int cl = ec[lo], rb = j - eb[lo];
+      const int nbl = (cl + kGroup - 1) / kGroup;
+      const int shift = rb == nbl - 1 ? pack_shift(cl - rb * kGroup) : 0;
+      // place inside the record's section, the section's start and size
+      const int64_t in = shift == 0 ? (int64_t)run_z + ez[lo] + rb
+                         : shift == 1 ? (int64_t)run_p1 + (ep[lo] & 0xffff) : (int64_t)run_p2 + (ep[lo] >> 16);
+      const int64_t first = shift == 0 ? 0 : shift == 1 ? (int64_t)b0 : (int64_t)b0 + b1;
+      const int size = shift == 0 ? b0 : shift == 1 ? b1 : b2;
+      if (in < size) {
+        PlanEntry pe;
+        pe.row0 = (uint32_t)(run_rows + er[lo] + (int64_t)rb * kGroup);
+        pe.rb = rb;
+        pe.count = cl;
+        pe.where = (shift == 0 ? kPlanUnpacked : shift == 1 ? kPlanPacked2 : kPlanPacked4) << 30 |
+                   (uint32_t)(run_blocks + j);
+        plan[first + in] = pe;
+      }
+    }
+    run_blocks += pass_blocks;
+    run_rows += er[T - 1] + ec[T - 1];
+    run_z += pass_z;
+    run_p1 += pass_p & 0xffff;
+    run_p2 += pass_p >> 16;
+    __syncthreads();
+  }
+  PlanEntry none;
+  none.row0 = 0;
+  none.rb = 0;
+  none.count = 0;
+  none.where = kPlanEmpty << 30;
+  for (int64_t at = (int64_t)run_z + t; at < b0; at += T) plan[at] = none;
+  for (int64_t at = (int64_t)b0 + run_p1 + t; at < (int64_t)b0 + b1; at += T) plan[at] = none;
+  for (int64_t at = (int64_t)b0 + b1 + run_p2 + t; at < (int64_t)b0 + b1 + b2; at += T) plan[at] = none;
+}
+
+// ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
+static BatchArgs batch_args(const void* counts, int counts_i64, int n_experts, const void* plan,
+                            const PlanShape* ps, bool packed_first) {
+  if (plan != nullptr)
+    return BatchArgs{nullptr, 0, 0, 0, plan, (int)ps->unpacked, (int)ps->packed2, (int)ps->packed4, packed_first};
+  return BatchArgs{counts, counts_i64, n_experts, 0, nullptr, 0, 0, 0, 0};
+}
+
+int64_t expert_plan_bytes(const PlanShape& ps) { return ps.blocks() * (int64_t)sizeof(PlanEntry); }
+
+PlanShape expert_plan_shape(const int64_t* host_counts, int n_experts) {
+  PlanShape ps{0, 0, 0};
+  for (int e = 0; e < n_experts; ++e) {
+    const int64_t c = host_counts[e] > 0 ? host_counts[e] : 0;
+    const int64_t nb = (c + kGroup - 1) / kGroup;
+    if (nb == 0) continue;
+    const int last = (int)(c - (nb - 1) * kGroup);
+    const int shift = last <= 32 ? 2 : last <= 64 ? 1 : 0;  // pack_shift, on the host
+    ps.unpacked += nb - (shift > 0);
+    ps.packed2 += shift == 1;
+    ps.packed4 += shift == 2;
+  }
+  return ps;
+}
+
+hipError_t launch_expert_plan(const void* counts, int counts_i64, int n_experts, const PlanShape& ps, void* plan,
+                              hipStream_t stream) {
+  if (ps.blocks() == 0) return hipSuccess;
+  hipLaunchKernelGGL(expert_plan_kernel, dim3(1), dim3(1024), 0, stream, counts, counts_i64, n_experts,
+                     (int)ps.unpacked, (int)ps.packed2, (int)ps.packed4, (PlanEntry*)plan);
+  return hipGetLastError();
+}
+
 hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, int64_t M, int N,
                                   int round_scale, int mode, int kind, const void* counts, int counts_i64,
-                                  int n_experts, int64_t row_blocks, hipStream_t stream) {
+                                  int n_experts, int64_t row_blocks, hipStream_t stream, const void* plan,
+                                  const PlanShape* ps) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  BatchArgs b{counts, counts_i64, n_experts};
-  const int64_t tiles = row_blocks * (N / kGroup);
+  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstBlockwise);
+  const int64_t tiles = plan ? plan_workgroups(ps->unpacked, ps->packed2, ps->packed4, N / kGroup)
+                             : row_blocks * (N / kGroup);
   if (tiles == 0) return hipSuccess;
-  const bool batched = counts != nullptr;
+  const bool batched = counts != nullptr || plan != nullptr;
   const dim3 grid((unsigned)tiles),
       block(2048 / (batched ? Policy::kRowsPerThreadBlockwiseBatched : Policy::kRowsPerThreadBlockwise));
   FQ_DISPATCH_KIND(kind, K,
@@ -362,7 +492,7 @@ hipError_t launch_pad_permute_quant(const void* x, const void* indices, const vo
                                     int64_t M, int N, int round_scale, int kind, const void* counts, int counts_i64,
                                     int n_experts, int64_t row_blocks, hipStream_t stream) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  BatchArgs b{counts, counts_i64, n_experts, 16};
+  BatchArgs b{counts, counts_i64, n_experts, 16, nullptr, 0, 0, 0, 0};
   const int64_t tiles = row_blocks * (N / kGroup);
   if (tiles == 0) return hipSuccess;
   const dim3 grid((unsigned)tiles), block(256);
@@ -376,14 +506,15 @@ hipError_t launch_pad_permute_quant(const void* x, const void* indices, const vo
 hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_bf16, void* q, float* s, void* qt,
                                  float* st, int64_t M, int n, int round_scale, int mode, int kind,
                                  const void* counts, int counts_i64, int n_experts, int64_t row_blocks,
-                                 hipStream_t stream) {
+                                 hipStream_t stream, const void* plan, const PlanShape* ps) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  BatchArgs b{counts, counts_i64, n_experts};
+  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstSiluFwd);
   RowWeight w{weight, weight_bf16};
-  const int64_t tiles = row_blocks * (n / kGroup);
+  const int64_t tiles = plan ? plan_workgroups(ps->unpacked, ps->packed2, ps->packed4, n / kGroup)
+                             : row_blocks * (n / kGroup);
   if (tiles == 0) return hipSuccess;
   const dim3 grid((unsigned)tiles), block(2048 / Policy::kRowsPerThreadSiluFwd);
-  const bool batched = counts != nullptr;
+  const bool batched = counts != nullptr || plan != nullptr;
   const bool weighted = weight != nullptr;
   const bool all_full = !batched && M % kGroup == 0;
   FQ_DISPATCH_KIND(kind, K,
@@ -400,15 +531,15 @@ hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_b
 hipError_t launch_silu_quant_bwd(const void* g, const void* x, const void* weight, int weight_bf16, void* q,
                                  float* s, void* qt, float* st, float* dw_part, void* dw, int64_t M, int n,
                                  int round_scale, int kind, const void* counts, int counts_i64, int n_experts,
-                                 int64_t row_blocks, hipStream_t stream) {
+                                 int64_t row_blocks, hipStream_t stream, const void* plan, const PlanShape* ps) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  BatchArgs b{counts, counts_i64, n_experts};
+  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstSiluBwd);
   RowWeight w{weight, weight_bf16};
   const int nb = n / kGroup;
-  const int64_t tiles = row_blocks * nb;
+  const int64_t tiles = plan ? plan_workgroups(ps->unpacked, ps->packed2, ps->packed4, nb) : row_blocks * nb;
   if (tiles == 0) return hipSuccess;
   const dim3 grid((unsigned)tiles), block(512);
-  const bool batched = counts != nullptr;
+  const bool batched = counts != nullptr || plan != nullptr;
   FQ_DISPATCH_KIND(kind, K,
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_BOOL(batched, B,

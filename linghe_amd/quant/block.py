@@ -65,7 +65,7 @@ def triton_blockwise_quant(x, round_scale=False, output_mode=2, *, fp8_dtype=tor
 
 
 def triton_batch_blockwise_quant(xs, token_count_per_expert, splits, round_scale=False, *,
-                                 fp8_dtype=torch.float8_e4m3fn):
+                                 fp8_dtype=torch.float8_e4m3fn, plan=None):
     """
     per-expert blockwise quantisation (megatron flex MoE)
     Args:
@@ -73,6 +73,7 @@ def triton_batch_blockwise_quant(xs, token_count_per_expert, splits, round_scale
         token_count_per_expert: device int tensor [n_experts]
         splits: python int list of token_count_per_expert
         round_scale: whether round scale to power of 2
+        plan: optional linghe_amd.utils.silu.ExpertPlan built from the same counts
 
     Returns (flat, per-expert packed):
         x_q [bs, dim], x_scale (bs*dim/128,), xt_q (bs*dim,), xt_scale (blocks*dim,)
@@ -89,6 +90,14 @@ def triton_batch_blockwise_quant(xs, token_count_per_expert, splits, round_scale
     blocks = sum((int(c) + 127) // 128 for c in splits)
     xt_scale = torch.empty((blocks * N,), device=device, dtype=torch.float32)
     if M == 0:
+        return x_q, x_scale, xt_q, xt_scale
+    if plan is not None:
+        if plan.blocks != blocks or plan.table.device != device:
+            raise ValueError("plan does not belong to these splits / this device")
+        with _lib.on_device(device):
+            _lib.check(_lib.lib.fq_batched_blockwise_quant_planned(
+                _lib.ptr(xs), _lib.ptr(plan.table), plan.shape, _lib.ptr(x_q), _lib.ptr(x_scale), _lib.ptr(xt_q),
+                _lib.ptr(xt_scale), M, N, int(bool(round_scale)), _lib.fp8_kind(fp8_dtype), _lib.stream_of(xs)))
         return x_q, x_scale, xt_q, xt_scale
     counts = token_count_per_expert
     if counts.dtype == torch.int64:

@@ -14,6 +14,51 @@ def _blocks_of(splits) -> int:
     return sum((int(c) + 127) // 128 for c in splits)
 
 
+class ExpertPlan:
+    """Device-side table of the 128-row blocks of one set of per-expert counts.
+
+    The per-expert entry points find each workgroup's tile by a prefix scan over
+    ``counts``; handing them a plan (keyword ``plan``) replaces that scan by one
+    16-byte read and sizes the launch for exactly the workgroups that have a tile.
+    Build it once per set of counts (``build_expert_plan``) and reuse it for every
+    per-expert call of the layer: forward, backward, quantiser.  No counterpart in
+    the reference, whose kernels are launched on a grid derived from the host-side
+    ``splits`` instead.
+    """
+
+    __slots__ = ("table", "shape", "blocks")
+
+    def __init__(self, table: torch.Tensor, shape):
+        self.table = table
+        self.shape = shape            # ctypes int64[4]: row blocks, whole / halved / quartered ones
+        self.blocks = int(shape[0])
+
+
+def build_expert_plan(counts: torch.Tensor, splits) -> ExpertPlan:
+    """counts: device int32/int64 [n_experts]; splits: the same numbers as a python list."""
+    import ctypes
+
+    n = len(splits)
+    host = (ctypes.c_int64 * max(n, 1))(*[int(c) for c in splits])
+    shape = (ctypes.c_int64 * 4)()
+    _lib.check(_lib.lib.fq_expert_plan_shape(host, n, shape))
+    nbytes = int(_lib.lib.fq_expert_plan_bytes(shape))
+    table = torch.empty((max(nbytes, 16),), device=counts.device, dtype=torch.uint8)
+    if shape[0]:
+        with _lib.on_device(counts.device):
+            _lib.check(_lib.lib.fq_build_expert_plan(
+                _lib.ptr(counts), _counts_flag(counts), counts.shape[0], shape, _lib.ptr(table),
+                _lib.stream_of(counts)))
+    return ExpertPlan(table, shape)
+
+
+def _check_plan(plan: ExpertPlan, blocks: int, device) -> None:
+    if plan.blocks != blocks:
+        raise ValueError(f"plan was built for {plan.blocks} row blocks, splits give {blocks}")
+    if plan.table.device != device:
+        raise ValueError("plan lives on another device")
+
+
 def _counts_flag(counts: torch.Tensor) -> int:
     if counts.dtype == torch.int64:
         return 1
@@ -174,6 +219,7 @@ def triton_batch_weighted_silu_and_block_quant_forward(
     output_mode=2,
     *,
     fp8_dtype=torch.float8_e4m3fn,
+    plan=None,
 ):
     """
     silu and blockwise quantize activation in routed experts
@@ -184,6 +230,7 @@ def triton_batch_weighted_silu_and_block_quant_forward(
         splits: python int list of token count per expert
         round_scale: whether round scale to power of 2
         output_mode: one of {0, 1, 2}
+        plan: optional ExpertPlan built from the same counts (same results, no scan of the counts)
 
     Returns (per-expert packed layouts):
         - out: quantized tensor [M, n]
@@ -211,6 +258,14 @@ def triton_batch_weighted_silu_and_block_quant_forward(
     transpose_scale = torch.empty((blocks, n), device=device, dtype=torch.float32)
     if M == 0:
         return out, scale, transpose_output, transpose_scale
+    if plan is not None:
+        _check_plan(plan, blocks, device)
+        with _lib.on_device(device):
+            _lib.check(_lib.lib.fq_batched_swiglu_quant_fwd_planned(
+                _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(plan.table), plan.shape,
+                _lib.ptr(out), _lib.ptr(scale), _lib.ptr(transpose_output), _lib.ptr(transpose_scale), M, n,
+                int(bool(round_scale)), output_mode, _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
+        return out, scale, transpose_output, transpose_scale
     with _lib.on_device(device):
         _lib.check(_lib.lib.fq_batched_swiglu_quant_fwd(
             _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(counts), _counts_flag(counts),
@@ -221,10 +276,11 @@ def triton_batch_weighted_silu_and_block_quant_forward(
 
 
 def triton_batch_weighted_silu_and_block_quant_backward(
-    g, x, weight, counts, splits=None, round_scale=False, *, fp8_dtype=torch.float8_e4m3fn
+    g, x, weight, counts, splits=None, round_scale=False, *, fp8_dtype=torch.float8_e4m3fn, plan=None
 ):
     """
     backward of triton_batch_weighted_silu_and_block_quant_forward
+    (plan: optional ExpertPlan built from the same counts)
     Returns:
         - dx: quantized non-transposed gradient [M, 2n]
         - dx_scale: per-expert packed scales, allocated [M, 2n/128]
@@ -251,6 +307,15 @@ def triton_batch_weighted_silu_and_block_quant_backward(
     if s == 0:
         return dx, dx_scale, dw, transpose_dx, transpose_dx_scale
     dws = torch.empty((M, n // 128), device=device, dtype=torch.float32)
+    if plan is not None:
+        _check_plan(plan, s, device)
+        with _lib.on_device(device):
+            _lib.check(_lib.lib.fq_batched_swiglu_quant_bwd_planned(
+                _lib.ptr(g), _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(plan.table), plan.shape,
+                _lib.ptr(dx), _lib.ptr(dx_scale), _lib.ptr(dw), _lib.ptr(transpose_dx),
+                _lib.ptr(transpose_dx_scale), _lib.ptr(dws), M, n, int(bool(round_scale)),
+                _lib.fp8_kind(fp8_dtype), _lib.stream_of(x)))
+        return dx, dx_scale, dw, transpose_dx, transpose_dx_scale
     with _lib.on_device(device):
         _lib.check(_lib.lib.fq_batched_swiglu_quant_bwd(
             _lib.ptr(g), _lib.ptr(x), _lib.ptr(weight), _weight_flag(weight), _lib.ptr(counts),

@@ -175,8 +175,8 @@ def test_entry_points_keep_reference_signatures(ref):
     positional = [p.name for p in sig.parameters.values() if p.kind == p.POSITIONAL_OR_KEYWORD]
     assert positional == params, (ref, positional)
     extras = [p.name for p in sig.parameters.values() if p.kind == p.KEYWORD_ONLY]
-    # additions are keyword-only: the FP8 format, and the caller-packed router weight
-    assert set(extras) <= {"fp8_dtype", "packed_route_weight"}
+    # additions are keyword-only: the FP8 format, the caller-packed router weight, and the per-expert tile plan
+    assert set(extras) <= {"fp8_dtype", "packed_route_weight", "plan"}
 
 
 def test_host_asserts_fire_on_cpu_tensors():
@@ -235,3 +235,45 @@ def test_facade_contract_helpers():
     assert codes.row.shape == (6, 5, 128) and codes.col.shape == (128, 6, 5) and codes.row_scale is None
     none = act.unfold(Codes(None, None, None, None), 128)
     assert none.row is None and none.col is None
+
+
+def test_expert_plan_shape_on_host():
+    """fq_expert_plan_shape is host arithmetic on the caller's copy of the counts: row blocks in
+    all, and how many are worked on whole, in halves (a last block of 33..64 rows) and in quarters
+    (at most 32 rows).  The planned entry points refuse anything that is not such a shape."""
+    from linghe_amd import _lib
+
+    L = _lib.lib
+    cases = {
+        (): [0, 0, 0, 0],
+        (0, 0): [0, 0, 0, 0],
+        (128,): [1, 1, 0, 0],
+        (129,): [2, 1, 0, 1],
+        (32, 33, 64, 65): [4, 1, 2, 1],
+        # 128+128+44 | - | 1 | 127 | 128+64 | 106*128+49
+        (300, 0, 1, 127, 192, 13617): [3 + 1 + 1 + 2 + 107, 2 + 1 + 1 + 106, 3, 1],
+    }
+    for counts, want in cases.items():
+        host = (ctypes.c_int64 * max(len(counts), 1))(*counts)
+        shape = (ctypes.c_int64 * 4)(-1, -1, -1, -1)
+        assert L.fq_expert_plan_shape(host, len(counts), shape) == 0
+        assert list(shape) == want, (counts, list(shape))
+        assert L.fq_expert_plan_bytes(shape) == 16 * want[0]
+    assert L.fq_expert_plan_shape(None, 3, shape) == -1
+    bad = (ctypes.c_int64 * 4)(5, 1, 1, 1)  # the parts do not add up
+    rc = L.fq_batched_blockwise_quant_planned(None, ctypes.c_void_p(256), bad, None, None, None, None, 640, 128, 0, 0,
+                                              None)
+    assert rc == -2 and b"plan shape" in L.fq_last_error()
+    assert L.fq_build_expert_plan(None, 0, 4, bad, ctypes.c_void_p(256), None) == -2
+    good = (ctypes.c_int64 * 4)(3, 1, 1, 1)
+    # more row blocks than rows
+    rc = L.fq_batched_swiglu_quant_fwd_planned(ctypes.c_void_p(256), ctypes.c_void_p(256), 0, ctypes.c_void_p(256),
+                                               good, ctypes.c_void_p(256), ctypes.c_void_p(256), ctypes.c_void_p(256),
+                                               ctypes.c_void_p(256), 2, 128, 0, 2, 0, None)
+    assert rc == -2 and b"inconsistent" in L.fq_last_error()
+    # no plan
+    rc = L.fq_batched_swiglu_quant_bwd_planned(ctypes.c_void_p(256), ctypes.c_void_p(256), ctypes.c_void_p(256), 0,
+                                               None, good, ctypes.c_void_p(256), ctypes.c_void_p(256),
+                                               ctypes.c_void_p(256), ctypes.c_void_p(256), ctypes.c_void_p(256),
+                                               ctypes.c_void_p(256), 640, 128, 0, 0, None)
+    assert rc == -1 and b"plan NULL" in L.fq_last_error()
