@@ -78,6 +78,13 @@ struct Policy {
   static constexpr bool kPlanPackedFirstSiluFwd = false;
   static constexpr bool kPlanPackedFirstSiluBwd = false;
   static constexpr bool kPlanPackedFirstBlockwise = true;
+  // row blocks per run that an XCD works on (xcd_runs; 0: every eighth tile).  Same sizes, planned launches with
+  // 0 / 2 / 4 / 8 / 16: SwiGLU forward 43.4 / 41.2 / 40.8 / 40.7 / 40.8 us, backward 76.5 / 76.1 / 75.5 / 75.3 / 76.2,
+  // blockwise quantiser 30.9 / 30.3 / 29.9 / 29.9 / 29.8.  Launches that scan the counts, 0 / 2 / 4 / 8: forward
+  // 44.4 / 45.2 / 45.1 / 45.6, backward 80.4 / 78.4 / 78.4 / 79.4, blockwise 31.1 / 32.2 / 32.4 / 32.7,
+  // gather + pad + quant 47.0 / 48.8 / 49.4 / 50.8: only the backward gains there
+  static constexpr int kXcdRowsPlanned = 8;
+  static constexpr int kXcdRowsSiluBwdCounts = 4;
   static constexpr bool kStartPriorityRmsnorm = true;
   // 16-byte chunks per lane, matrix and step in the bf16 SwiGLU backward (three matrices are read):
   // 29.0 / 30.4 / 28.7 / 35.5 us with 2 / 3 / 4 / 8 at 8192 x 4096

@@ -31,6 +31,7 @@ struct BatchArgs {
   int plan_unpacked;   // records of row blocks that are worked on unpacked,
   int plan_packed2;    // of last blocks of 33..64 rows, and (behind them) of
   int plan_packed4;    // last blocks of at most 32 rows: the table's three sections, counted by the host
+  int xcd_rows;        // > 0: every XCD works on runs of so many row blocks (xcd_runs)
   int plan_packed_first;  // order of a planned launch: the packed tiles before (1) or behind (0) the others
 };
 
@@ -58,6 +59,22 @@ static_assert(sizeof(PlanEntry) == 16, "16-byte records");
 // workgroups of a planned launch over ncb column blocks
 __host__ __device__ inline int64_t plan_workgroups(int64_t unpacked, int64_t packed2, int64_t packed4, int ncb) {
   return unpacked * ncb + packed2 * ((ncb + 1) >> 1) + packed4 * ((ncb + 3) >> 2);
+}
+
+// Workgroup i runs on XCD i % 8, each with an L2 of its own.  Neighbouring row blocks of an expert
+// share lines of the transposed outputs (a column's 128-byte run starts at any byte offset), which
+// one L2 merges and two write out twice as partial lines.  This renumbering hands every XCD runs
+// of `chunk` consecutive tiles (a few row blocks with all their column blocks) instead of every
+// eighth tile, in rounds of 8 * chunk tiles so that the XCDs stay in step; the tiles behind the
+// last full round keep their numbers.
+__device__ __forceinline__ int xcd_runs(int id, int total, int chunk) {
+  const int round_tiles = 8 * chunk;
+  if (id < (total / round_tiles) * round_tiles) {
+    const int xcd = id & 7, pos = id >> 3;
+    const int round = pos / chunk;
+    return (round * 8 + xcd) * chunk + (pos - round * chunk);
+  }
+  return id;
 }
 
 // out_w: width of the quantised matrix the tile belongs to (n, or 2n for the
@@ -122,7 +139,8 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
       x = r - q * c2;
       kind = kPlanPacked4;
     } else {
-      const int r = id - n1 - n2;
+      int r = id - n1 - n2;
+      if (b.xcd_rows > 0) r = xcd_runs(r, b.plan_unpacked * ncb, b.xcd_rows * ncb);
       idx = r / ncb;
       x = r - idx * ncb;
     }
@@ -148,6 +166,7 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
     g.st_row = (int64_t)(where & 0x3fffffffu);
     if (g.row0 + g.rows_store > M) g.valid = false;
   } else {
+    if (b.xcd_rows > 0) id = xcd_runs(id, (int)n_wg_x(), b.xcd_rows * ncb);
     const ExpertTile et = find_expert_tile(b.counts, b.counts_i64, b.n_experts, id, ncb, b.pad > 1 ? b.pad : 1);
     // the lookup's answer is the same in every lane: keep it in scalar registers
     const int expert = uniform32(et.expert), count = uniform32(et.count), rb = uniform32(et.rb);

@@ -305,7 +305,7 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadRmsnorm) void rmsnorm_
   // lets the newcomers push aside the stores of the ones at work: 4 % slower at 16384 x 7168.
   if (first) __builtin_amdgcn_s_setprio(3);
   __shared__ TileShared<RPT> sh;
-  BatchArgs none{nullptr, 0, 0, 0, nullptr, 0, 0, 0, 0};
+  BatchArgs none{nullptr, 0, 0, 0, nullptr, 0, 0, 0, 0, 0};
   const TileGeom g = resolve_tile<false>(M, n / kGroup, n, none, remap);
   if (!g.valid) return;
   uint4 raw[RPT];
@@ -435,10 +435,11 @@ __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restric
 // launchers
 // ---------------------------------------------------------------------------
 static BatchArgs batch_args(const void* counts, int counts_i64, int n_experts, const void* plan,
-                            const PlanShape* ps, bool packed_first) {
+                            const PlanShape* ps, bool packed_first, int xcd_rows_scan) {
   if (plan != nullptr)
-    return BatchArgs{nullptr, 0, 0, 0, plan, (int)ps->unpacked, (int)ps->packed2, (int)ps->packed4, packed_first};
-  return BatchArgs{counts, counts_i64, n_experts, 0, nullptr, 0, 0, 0, 0};
+    return BatchArgs{nullptr, 0, 0, 0, plan, (int)ps->unpacked, (int)ps->packed2, (int)ps->packed4,
+                     Policy::kXcdRowsPlanned, packed_first};
+  return BatchArgs{counts, counts_i64, n_experts, 0, nullptr, 0, 0, 0, xcd_rows_scan, 0};
 }
 
 int64_t expert_plan_bytes(const PlanShape& ps) { return ps.blocks() * (int64_t)sizeof(PlanEntry); }
@@ -471,7 +472,7 @@ hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, fl
                                   int n_experts, int64_t row_blocks, hipStream_t stream, const void* plan,
                                   const PlanShape* ps) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstBlockwise);
+  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstBlockwise, 0);
   const int64_t tiles = plan ? plan_workgroups(ps->unpacked, ps->packed2, ps->packed4, N / kGroup)
                              : row_blocks * (N / kGroup);
   if (tiles == 0) return hipSuccess;
@@ -492,7 +493,7 @@ hipError_t launch_pad_permute_quant(const void* x, const void* indices, const vo
                                     int64_t M, int N, int round_scale, int kind, const void* counts, int counts_i64,
                                     int n_experts, int64_t row_blocks, hipStream_t stream) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  BatchArgs b{counts, counts_i64, n_experts, 16, nullptr, 0, 0, 0, 0};
+  BatchArgs b{counts, counts_i64, n_experts, 16, nullptr, 0, 0, 0, 0, 0};
   const int64_t tiles = row_blocks * (N / kGroup);
   if (tiles == 0) return hipSuccess;
   const dim3 grid((unsigned)tiles), block(256);
@@ -508,7 +509,7 @@ hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_b
                                  const void* counts, int counts_i64, int n_experts, int64_t row_blocks,
                                  hipStream_t stream, const void* plan, const PlanShape* ps) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstSiluFwd);
+  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstSiluFwd, 0);
   RowWeight w{weight, weight_bf16};
   const int64_t tiles = plan ? plan_workgroups(ps->unpacked, ps->packed2, ps->packed4, n / kGroup)
                              : row_blocks * (n / kGroup);
@@ -533,7 +534,8 @@ hipError_t launch_silu_quant_bwd(const void* g, const void* x, const void* weigh
                                  int round_scale, int kind, const void* counts, int counts_i64, int n_experts,
                                  int64_t row_blocks, hipStream_t stream, const void* plan, const PlanShape* ps) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
-  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstSiluBwd);
+  const BatchArgs b = batch_args(counts, counts_i64, n_experts, plan, ps, Policy::kPlanPackedFirstSiluBwd,
+                                   Policy::kXcdRowsSiluBwdCounts);
   RowWeight w{weight, weight_bf16};
   const int nb = n / kGroup;
   const int64_t tiles = plan ? plan_workgroups(ps->unpacked, ps->packed2, ps->packed4, nb) : row_blocks * nb;
