@@ -532,6 +532,30 @@ def build_cases(names, dev):
     # a wide router: more than 512 logits run as one launch per 512 (virtual) columns, x re-read by each
     add("next_router_wide", build=lambda: router_case(False, (2048, 2048, 2048), "next_router_wide"))
 
+    # ---------------------------------------------------------------- the per-expert tile plan of cfg3's counts
+    def plan_case():
+        import ctypes
+        d = lazy.setdefault("cfg3", configs.cfg3_batched_swiglu())
+        counts = d["counts"]
+        cnt = torch.tensor(counts, dtype=torch.int32, device=dev)
+        host = (ctypes.c_int64 * len(counts))(*counts)
+        shape = (ctypes.c_int64 * 4)()
+        _lib.check(L.fq_expert_plan_shape(host, len(counts), shape))
+        nbytes = int(L.fq_expert_plan_bytes(shape))
+
+        def make_set():
+            s = dict(plan=torch.empty((nbytes,), device=dev, dtype=torch.uint8))
+            s["args"] = (_p(cnt), 0, len(counts), shape, _p(s["plan"]), stream)
+            return s
+
+        def launch(s):
+            _lib.check(L.fq_build_expert_plan(*s["args"]))
+
+        return Case("expert_plan", "fq_build_expert_plan (one launch per set of counts)", [len(counts)],
+                    (4 * len(counts), nbytes), make_set, launch, None)
+
+    add("expert_plan", build=plan_case)
+
     # ---------------------------------------------------------------- the no-work stream kernel on a known size
     # (the read / copy rates of the memory system, and the calibration of FETCH_SIZE / WRITE_SIZE)
     def stream_case(name, read_mib, write_mib):
@@ -777,7 +801,7 @@ def load_traffic_table():
 
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
        "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg5b_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
-       "cfg3_planned", "cfg3b_planned", "a8_batch_blockwise_planned",
+       "cfg3_planned", "cfg3b_planned", "a8_batch_blockwise_planned", "expert_plan",
        "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed", "next_router_wide",
        "stream_read", "stream_copy"]
 

@@ -500,12 +500,12 @@ __device__ __forceinline__ void load_counts(const void* counts, int is_i64, int 
 // barriers cost 13 % of the batched SwiGLU forward, one wave scanning for the others 6 %.)
 // A workgroup beyond the last tile (the launch is sized for one workgroup per 128 x 128 tile,
 // packing needs fewer) or counts that disagree with the host's yield expert = -1.
-// Tiles are taken in grid order.  (Numbering them so that every XCD works on one contiguous
-// eighth of the real tiles - neighbouring row blocks of an expert share lines of the transposed
-// output, which one L2 merges and two do not: 11 % fewer bytes written by the per-expert SwiGLU
-// backward - needs the number of tiles first, one more pass over the counts, and measured
-// slower: 89.3 against 87.8 us for that kernel at 65536 x 1024 with 256 experts, 59 against
-// 51 us for gather+pad+quant.)
+// `wg` is the tile's number in that order; which workgroup takes which number is the caller's
+// choice (resolve_tile: grid order, or runs of neighbouring row blocks per XCD).  Numbering the
+// tiles so that every XCD works on one contiguous eighth of the REAL tiles needs their number
+// first, one more pass over the counts, and measured slower: 89.3 against 87.8 us for the
+// per-expert SwiGLU backward at 65536 x 1024 with 256 experts, 59 against 51 us for
+// gather+pad+quant.
 // pad > 1: every expert's region starts at a multiple of pad rows (the reference's
 // permute-and-pad layout, pad = 16); 128 is a multiple of pad, so the number of
 // 128-row blocks of an expert does not change.

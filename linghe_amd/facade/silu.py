@@ -51,16 +51,17 @@ class BlockBatchWeightedSiluFunction(torch.autograd.Function):
     `splits` the same numbers on the host), `weights` is one router probability per
     row.  Outputs keep the kernels' per-expert packing, so nothing is re-viewed.
     The quantizer lists are passed through to the tensor class; their first member
-    gives the scale rounding and the FP8 format of all experts."""
+    gives the scale rounding and the FP8 format of all experts.  `plan` (optional, an
+    ExpertPlan of the same counts) is handed to the forward and kept for the backward."""
 
     @staticmethod
-    def forward(ctx, input, weights, counts, splits, quantizers, grad_quantizers, cls, is_recomputing):
+    def forward(ctx, input, weights, counts, splits, quantizers, grad_quantizers, cls, is_recomputing, plan=None):
         lead = quantizers[0]
         ctx.save_for_backward(input, weights, counts)
-        ctx.sidecar = (splits, grad_quantizers, cls, input.requires_grad)
+        ctx.sidecar = (splits, grad_quantizers, cls, input.requires_grad, plan)
         got = triton_batch_weighted_silu_and_block_quant_forward(
             input, weights, counts, splits=splits, round_scale=lead.force_pow_2_scales,
-            output_mode=output_mode(is_recomputing), fp8_dtype=kernel_fp8_dtype(lead.dtype))
+            output_mode=output_mode(is_recomputing), fp8_dtype=kernel_fp8_dtype(lead.dtype), plan=plan)
         codes = Codes(*got)
         return wrap(cls, codes, shape=codes.row.shape, dtype=input.dtype, quantizer=quantizers,
                     fp8_tag=lead.dtype, requires_grad=input.requires_grad)
@@ -68,19 +69,19 @@ class BlockBatchWeightedSiluFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         input, weights, counts = ctx.saved_tensors
-        splits, grad_quantizers, cls, needs_grad = ctx.sidecar
+        splits, grad_quantizers, cls, needs_grad, plan = ctx.sidecar
         lead = grad_quantizers[0]
         dq, dq_scale, dweights, dqt, dqt_scale = triton_batch_weighted_silu_and_block_quant_backward(
             grad_output.contiguous(), input, weights, counts, splits=splits,
-            round_scale=lead.force_pow_2_scales, fp8_dtype=kernel_fp8_dtype(lead.dtype))
+            round_scale=lead.force_pow_2_scales, fp8_dtype=kernel_fp8_dtype(lead.dtype), plan=plan)
         dx = wrap(cls, Codes(dq, dq_scale, dqt, dqt_scale), shape=input.shape, dtype=grad_output.dtype,
                   quantizer=grad_quantizers, fp8_tag=lead.dtype, requires_grad=needs_grad)
-        # one gradient slot per forward argument: input, weights, then six non-tensors
-        return (dx, dweights) + (None,) * 6
+        # one gradient slot per forward argument: input, weights, then seven non-tensors
+        return (dx, dweights) + (None,) * 7
 
 
 def block_batch_weighted_silu_impl(input, weights, counts, splits, quantizers, grad_quantizers, cls,
-                                   is_recomputing=None):
+                                   is_recomputing=None, *, plan=None):
     assert input.ndim == 2
     return BlockBatchWeightedSiluFunction.apply(input, weights, counts, splits, quantizers, grad_quantizers,
-                                                cls, is_recomputing)
+                                                cls, is_recomputing, plan)

@@ -176,11 +176,13 @@ def test_block_silu(gpu, pow2, gdtype, gtag):
                      gk["columnwise_scale_inv"], **tolb)
 
 
+@pytest.mark.parametrize("with_plan", [False, True])
 @pytest.mark.parametrize("is_recomputing,gdtype", [(None, E4M3), (False, E4M3), (True, E4M3), (None, E5M2)])
-def test_block_batch_weighted_silu(gpu, is_recomputing, gdtype):
+def test_block_batch_weighted_silu(gpu, is_recomputing, gdtype, with_plan):
     from linghe_amd.facade.silu import block_batch_weighted_silu_impl
+    from linghe_amd.utils.silu import build_expert_plan
 
-    announce("facade BlockBatchWeightedSiluFunction", is_recomputing, gdtype)
+    announce("facade BlockBatchWeightedSiluFunction", is_recomputing, gdtype, with_plan)
     counts = [160, 0, 96, 272, 16, 128, 33, 64]
     bs, N = sum(counts), 1024
     g = gen(54)
@@ -193,8 +195,10 @@ def test_block_batch_weighted_silu(gpu, is_recomputing, gdtype):
     cnt = torch.tensor(counts, dtype=torch.int32, device=gpu)
     qs = [Quantizer() for _ in counts]
     gqs = [Quantizer(dtype=gdtype) for _ in counts]
+    # a tile plan built once from the counts serves the forward and, kept by the function, the backward
+    plan = build_expert_plan(cnt, counts) if with_plan else None
     out = block_batch_weighted_silu_impl(Capture.apply(leaf), wd, cnt, counts, qs, gqs, FakeQTensor,
-                                         is_recomputing=is_recomputing)
+                                         is_recomputing=is_recomputing, plan=plan)
     torch.cuda.synchronize()
     assert isinstance(out, FakeQTensor) and tuple(out.shape) == (bs, N // 2)
     kw = out.kw
