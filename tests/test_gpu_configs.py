@@ -126,6 +126,18 @@ def test_cfg3_batched_swiglu_full(gpu):
     check_quant_pair("cfg3.bwd.row", rb[0], rb[1], dq, ds.view(-1), **FUSED_BWD)
     check_quant_pair("cfg3.bwd.col", rb[3], rb[4], dqt.view(-1), dst.view(-1), **FUSED_BWD)
     torch.testing.assert_close(dw.cpu(), rb[2], rtol=1e-4, atol=1e-4 * float(rb[2].abs().max()))
+    # the same calls with the tiles read from a plan: every output byte for byte
+    from linghe_amd.quant.block import triton_batch_blockwise_quant
+    from linghe_amd.utils.silu import build_expert_plan
+
+    plan = build_expert_plan(cnt, counts)
+    planned = fwd(xd, wd, cnt, counts, output_mode=2, plan=plan) + bwd(dyd, xd, wd, cnt, splits=counts, plan=plan)
+    torch.cuda.synchronize()
+    for a, b in zip((q, s, qt, st, dq, ds, dw, dqt, dst), planned):
+        assert _same_bits(a.cpu(), b.cpu())
+    y = dyd  # 65536 x 512 bf16: the per-expert quantiser on a matrix of the activations' shape
+    for a, b in zip(triton_batch_blockwise_quant(y, cnt, counts), triton_batch_blockwise_quant(y, cnt, counts, plan=plan)):
+        assert _same_bits(a.cpu(), b.cpu())
 
 
 @pytest.mark.parametrize("dtype", [E4M3, E5M2])
