@@ -43,6 +43,11 @@ int64_t expert_plan_bytes(const PlanShape& ps);
 hipError_t launch_expert_plan(const void* counts, int counts_i64, int n_experts, const PlanShape& ps, void* plan,
                               hipStream_t stream);
 
+// RMSNorm + quant with both outputs runs the statistic pass (launch_rmsnorm_fwd, quant = 2) and then
+// the tile kernel (launch_rmsnorm_quant_tile, mode 2); for these shapes both hand XCD X the X-th
+// eighth of the rows, so that the second pass finds in its XCD's L2 what the first one left there
+bool rmsnorm_passes_by_xcd(int64_t M, int n);
+
 hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const float* rstd, void* q, float* s,
                                      void* qt, float* st, int64_t M, int n, int round_scale, int mode, int kind,
                                      hipStream_t stream);

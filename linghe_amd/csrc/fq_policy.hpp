@@ -86,6 +86,14 @@ struct Policy {
   static constexpr int kXcdRowsPlanned = 8;
   static constexpr int kXcdRowsSiluBwdCounts = 4;
   static constexpr bool kStartPriorityRmsnorm = true;
+  // RMSNorm + quant in two passes, both passes giving XCD X (workgroup number mod 8) the X-th eighth of the rows,
+  // the statistic pass walking its eighth from the end and the tile kernel from the start: what the tile kernel
+  // reads first is what the same XCD's L2 read last.  Rows a multiple of 1024 (the eighths are whole row blocks).
+  // us without / with: 2048 x 2048 8.8 / 7.9, 4096 x 2048 11.7 / 10.6, 8192 x 2048 17.9 / 16.6, 3072 x 4096
+  // 14.6 / 13.3, 4096 x 7168 30.2 / 27.9, 8192 x 4096 33.0 / 32.0, 16384 x 2048 33.2 / 31.7, 8192 x 7168
+  // 55.8 / 52.9, 16384 x 4096 63.4 / 62.7, 32768 x 2048 63.6 / 63.3, 16384 x 7168 108.1 / 109.6: up to this
+  // many bytes of input
+  static constexpr long long kRmsnormByXcdMaxBytes = 160ll << 20;
   // 16-byte chunks per lane, matrix and step in the bf16 SwiGLU backward (three matrices are read):
   // 29.0 / 30.4 / 28.7 / 35.5 us with 2 / 3 / 4 / 8 at 8192 x 4096
   static constexpr int kSwigluBwdRowsUnroll = 4;

@@ -251,7 +251,7 @@ __global__ __launch_bounds__(T) void rmsnorm_fwd_kernel(const uint16_t* __restri
 // reads the row's last chunk again and counts as zero.
 template <int U>
 __global__ __launch_bounds__(64 * Policy::kRowstatWaves) void rowstat_kernel(const uint16_t* __restrict__ x, float* __restrict__ rstd,
-                                                     int64_t M, int n, float eps) {
+                                                     int64_t M, int n, float eps, int by_xcd) {
   constexpr int kW = Policy::kRowstatWaves;  // waves (rows) per workgroup
   const int lane = tid_x() & 63;
   const int chunks = n >> 3;
@@ -259,8 +259,14 @@ __global__ __launch_bounds__(64 * Policy::kRowstatWaves) void rowstat_kernel(con
   // walks the matrix forwards, so it starts with the rows this kernel read last, which
   // are the ones still in the last-level cache: for an input about the size of that
   // cache roughly half of the second read never reaches HBM.
-  for (int64_t k = (int64_t)wg_x() * kW + (tid_x() >> 6); k < M; k += (int64_t)n_wg_x() * kW) {
-    const int64_t row = M - 1 - k;
+  // by_xcd: workgroup w runs on XCD w % 8, and XCD X takes the X-th eighth of the rows, again from its
+  // end backwards: the tile kernel hands the same eighth to the same XCD (rmsnorm_passes_by_xcd)
+  const int64_t span = by_xcd ? M >> 3 : M;
+  const int64_t first = by_xcd ? (int64_t)(wg_x() & 7) * span : 0;
+  const int64_t k0 = by_xcd ? (int64_t)(wg_x() >> 3) * kW + (tid_x() >> 6) : (int64_t)wg_x() * kW + (tid_x() >> 6);
+  const int64_t step = by_xcd ? (int64_t)(n_wg_x() >> 3) * kW : (int64_t)n_wg_x() * kW;
+  for (int64_t k = k0; k < span; k += step) {
+    const int64_t row = first + span - 1 - k;
     const uint4* p = (const uint4*)(x + row * n);
     double ss = 0.0;
     for (int c0 = 0; c0 < chunks; c0 += U * 64) {
@@ -617,8 +623,9 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
   // quant: 0 = bf16 output, 1 = fp8 codes + scales, 2 = statistic only (its own kernel)
   if (quant == 2) {
     const dim3 sgrid((unsigned)((wgs + Policy::kRowstatWaves - 1) / Policy::kRowstatWaves)), sblock(64 * Policy::kRowstatWaves);
-    if (n <= 2048) hipLaunchKernelGGL(rowstat_kernel<4>, sgrid, sblock, 0, stream, (const uint16_t*)x, rstd, M, n, eps);
-    else hipLaunchKernelGGL(rowstat_kernel<8>, sgrid, sblock, 0, stream, (const uint16_t*)x, rstd, M, n, eps);
+    const int by_xcd = rmsnorm_passes_by_xcd(M, n) && sgrid.x % 8 == 0;
+    if (n <= 2048) hipLaunchKernelGGL(rowstat_kernel<4>, sgrid, sblock, 0, stream, (const uint16_t*)x, rstd, M, n, eps, by_xcd);
+    else hipLaunchKernelGGL(rowstat_kernel<8>, sgrid, sblock, 0, stream, (const uint16_t*)x, rstd, M, n, eps, by_xcd);
   } else if (!quant) {
     if (reuse_rstd) { FQ_LAUNCH_FWD(true, 0, kE4M3, false) } else { FQ_LAUNCH_FWD(false, 0, kE4M3, false) }
   } else if (n > 2048) {
@@ -647,6 +654,10 @@ hipError_t launch_rmsnorm_fwd(const void* x, const void* gamma, void* out, float
   }
 #undef FQ_LAUNCH_FWD
   return hipGetLastError();
+}
+
+bool rmsnorm_passes_by_xcd(int64_t M, int n) {
+  return M % 1024 == 0 && M * n * 2 <= (int64_t)Policy::kRmsnormByXcdMaxBytes;
 }
 
 int64_t rmsnorm_bwd_partials(int64_t M) {

@@ -567,7 +567,8 @@ hipError_t launch_rmsnorm_quant_tile(const void* x, const void* gamma, const flo
   // transposed rows start every M bytes: off 16-byte boundaries their stores go out plain
   const bool aligned_rows = M % 16 == 0;
   // XCD remap (see resolve_tile): wide rows and several waves of workgroups
-  const int remap = aligned_rows && n >= 4096 && tiles >= 3072;
+  // ... and, behind the statistic pass, wherever that pass handed out the rows by XCD
+  const int remap = (aligned_rows && n >= 4096 && tiles >= 3072) || (mode == 2 && rmsnorm_passes_by_xcd(M, n));
   // raised priority until the loads are out: only when the whole launch is resident at once (four
   // workgroups per CU of a 256-CU device; more tiles than that arrive in generations)
   const int first = Policy::kStartPriorityRmsnorm && tiles <= 1024;
