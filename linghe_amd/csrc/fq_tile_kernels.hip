@@ -14,7 +14,9 @@ namespace fq {
 // ---------------------------------------------------------------------------
 // plain blockwise quant
 // ---------------------------------------------------------------------------
-template <int KIND, bool ROUND, int MODE, bool BATCHED>
+// PLANNED: the per-expert form with its tiles read from a plan (same code; another cache policy,
+// because its tile numbering lets an XCD's L2 merge the partial lines of the transposed codes)
+template <int KIND, bool ROUND, int MODE, bool BATCHED, bool PLANNED = false>
 __global__ __launch_bounds__(2048 / (BATCHED ? Policy::kRowsPerThreadBlockwiseBatched : Policy::kRowsPerThreadBlockwise))
 void blockwise_quant_kernel(const uint16_t* __restrict__ x, OutPtrs out, int64_t M, int N, BatchArgs batch) {
   constexpr int RPT = BATCHED ? Policy::kRowsPerThreadBlockwiseBatched : Policy::kRowsPerThreadBlockwise;
@@ -23,7 +25,8 @@ void blockwise_quant_kernel(const uint16_t* __restrict__ x, OutPtrs out, int64_t
   if (!g.valid) return;
   uint4 raw[RPT];
   constexpr bool LDNT = BATCHED ? Policy::kLoadHintBlockwiseBatched : Policy::kLoadHintBlockwise;
-  constexpr int NT = BATCHED ? Policy::kStoreHintBlockwiseBatched : Policy::kStoreHintBlockwise;
+  constexpr int NT = PLANNED ? Policy::kStoreHintBlockwisePlanned
+                     : BATCHED ? Policy::kStoreHintBlockwiseBatched : Policy::kStoreHintBlockwise;
   constexpr bool LEAN = BATCHED || Policy::kLeanBlockwise;
   const TilePart<RPT> tp = tile_part<RPT>(g);
   load_rows<RPT, LDNT, LEAN>(x + g.row0 * N + (int64_t)(g.cb + tp.asub) * kGroup, N, tp.rows, raw, tp.sl.rgl);
@@ -483,8 +486,9 @@ hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, fl
     FQ_DISPATCH_BOOL(round_scale, R,
       FQ_DISPATCH_MODE(mode, MD,
         FQ_DISPATCH_BOOL(batched, B,
-          hipLaunchKernelGGL((blockwise_quant_kernel<K, R, MD, B>), grid, block, 0, stream,
-                             (const uint16_t*)x, out, M, N, b);))))
+          FQ_DISPATCH_BOOL(plan != nullptr, P,
+            hipLaunchKernelGGL((blockwise_quant_kernel<K, R, MD, B || P, P>), grid, block, 0, stream,
+                               (const uint16_t*)x, out, M, N, b);)))))
   return hipGetLastError();
 }
 
