@@ -198,12 +198,12 @@ def build_cases(names, dev):
     add("cfg2_mode1", build=lambda: swiglu_fwd_case("cfg2_mode1", False, 1))
 
     # ---------------------------------------------------------------- cfg3 (+ backward)
-    def expert_plan(cnt, counts):
+    def expert_plan(cnt, counts, pad=1):
         """the per-expert tile plan of a set of counts (table, shape), built once outside the timed region"""
         import ctypes
         host = (ctypes.c_int64 * len(counts))(*counts)
-        shape = (ctypes.c_int64 * 4)()
-        _lib.check(L.fq_expert_plan_shape(host, len(counts), shape))
+        shape = (ctypes.c_int64 * 5)()
+        _lib.check(L.fq_expert_plan_shape(host, len(counts), pad, shape))
         table = torch.empty((max(int(L.fq_expert_plan_bytes(shape)), 16),), device=dev, dtype=torch.uint8)
         _lib.check(L.fq_build_expert_plan(_p(cnt), 0, len(counts), shape, _p(table), stream))
         return table, shape
@@ -336,8 +336,8 @@ def build_cases(names, dev):
     add("cfg5a", build=rms_bwd_case)
 
     # ---------------------------------------------------------------- next row: gather + pad + quant
-    def permute_case():
-        d = configs.next_permute_pad_quant()
+    def permute_case(planned=False):
+        d = lazy.setdefault("permute", configs.next_permute_pad_quant())
         x_cpu, probs_cpu, counts, idx_cpu = d["x"], d["probs"], d["counts"], d["indices"]
         m, N = x_cpu.shape
         M = idx_cpu.numel()
@@ -345,6 +345,7 @@ def build_cases(names, dev):
         blocks = sum((c + 127) // 128 for c in counts)
         cnt = torch.tensor(counts, dtype=torch.int32, device=dev)
         idx = idx_cpu.to(dev)
+        plan, pshape = expert_plan(cnt, counts, 16) if planned else (None, None)
 
         def make_set():
             s = dict(x=x_cpu.to(dev), probs=probs_cpu.to(dev), q=torch.empty((M, N), device=dev, dtype=FP8),
@@ -352,21 +353,26 @@ def build_cases(names, dev):
                      qt=torch.empty((M, N), device=dev, dtype=FP8),
                      st=torch.empty((blocks, N), device=dev, dtype=torch.float32),
                      p=torch.empty((M,), device=dev, dtype=torch.float32))
-            s["args"] = (_p(s["x"]), _p(cnt), 0, E, blocks, _p(idx), _p(s["probs"]), 0, _p(s["p"]), _p(s["q"]),
-                         _p(s["s"]), _p(s["qt"]), _p(s["st"]), m, M, N, 0, _lib.FQ_E4M3, stream)
+            src = (_p(plan), pshape, E) if planned else (_p(cnt), 0, E, blocks)
+            s["args"] = (_p(s["x"]),) + src + (_p(idx), _p(s["probs"]), 0, _p(s["p"]), _p(s["q"]), _p(s["s"]),
+                                              _p(s["qt"]), _p(s["st"]), m, M, N, 0, _lib.FQ_E4M3, stream)
             return s
 
+        fn = L.fq_batched_pad_permute_quant_planned if planned else L.fq_batched_pad_permute_quant
+
         def launch(s):
-            _lib.check(L.fq_batched_pad_permute_quant(*s["args"]))
+            _lib.check(fn(*s["args"]))
 
         def cpu_fn():
             from oracle import fq_oracle as O
             return O.batch_block_pad_permute_with_indices(x_cpu, d["indices_unpadded"], probs_cpu, counts, False)
 
-        return Case("next_permute", "triton_batch_block_pad_permute_with_indices", [M, N],
+        return Case("next_permute" + ("_planned" if planned else ""),
+                    "triton_batch_block_pad_permute_with_indices" + (" with plan=" if planned else ""), [M, N],
                     configs.rw_permute_pad_quant(N, counts), make_set, launch, cpu_fn)
 
     add("next_permute", build=permute_case)
+    add("next_permute_planned", build=lambda: permute_case(True))
 
     # ---------------------------------------------------------------- next rows: bf16 SwiGLU, weight block quant
     def wsilu_case(backward):
@@ -539,8 +545,8 @@ def build_cases(names, dev):
         counts = d["counts"]
         cnt = torch.tensor(counts, dtype=torch.int32, device=dev)
         host = (ctypes.c_int64 * len(counts))(*counts)
-        shape = (ctypes.c_int64 * 4)()
-        _lib.check(L.fq_expert_plan_shape(host, len(counts), shape))
+        shape = (ctypes.c_int64 * 5)()
+        _lib.check(L.fq_expert_plan_shape(host, len(counts), 1, shape))
         nbytes = int(L.fq_expert_plan_bytes(shape))
 
         def make_set():
@@ -802,7 +808,7 @@ def load_traffic_table():
 ALL = ["cfg1", "cfg2", "cfg3", "cfg3b", "cfg4", "cfg4_e5m2", "cfg5a", "cfg5b", "cfg5c",
        "cfg1_pow2", "cfg2_pow2", "cfg4_pow2", "cfg5b_pow2", "cfg1_mode0", "cfg5_mode0", "cfg1_mode1", "cfg2_mode0", "cfg2_mode1", "a2_rmsnorm_fwd", "a8_blockwise", "a8_group", "a8_batch_blockwise",
        "cfg3_planned", "cfg3b_planned", "a8_batch_blockwise_planned", "expert_plan",
-       "next_permute", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed", "next_router_wide",
+       "next_permute", "next_permute_planned", "next_wsilu_fwd", "next_wsilu_bwd", "next_block_quant", "next_router", "next_router_packed", "next_router_wide",
        "stream_read", "stream_copy"]
 
 

@@ -91,18 +91,21 @@ int fq_batched_blockwise_quant(const void* x, const void* counts, int counts_is_
  *  - fq_expert_plan_shape (host only, no GPU work) reads the caller's host-side
  *    copy of the counts - what the reference takes as `splits`
  *    (linghe/utils/silu.py:826, :838: "batch mode need splits to launch
- *    kernels") - and fills shape[0..3]: the number of 128-row blocks
- *    (= total_blocks of the other forms) and how many of them are worked on
- *    whole, in halves and in quarters;
- *  - fq_build_expert_plan writes one 16-byte record per row block from the
+ *    kernels") - and fills shape[0..4]: the number of 128-row blocks
+ *    (= total_blocks of the other forms), how many of them are worked on
+ *    whole, in halves and in quarters, and `pad`: 1 for the layouts in which
+ *    the experts lie back to back (SwiGLU, blockwise quantiser), 16 for the
+ *    gather + pad + quant layout (every expert's region rounded up to 16 rows);
+ *  - fq_build_expert_plan writes one 20-byte record per row block from the
  *    DEVICE-side counts into `plan` (fq_expert_plan_bytes(shape) bytes of
  *    device memory, 16-byte aligned);
  *  - the *_planned forms of the entry points take plan and shape in place of
  *    counts, n_experts and total_blocks.  Their outputs are identical to those
- *    of the forms that take the counts.  A plan addresses at most 2^31 - 1 rows.
+ *    of the forms that take the counts.  A plan addresses at most 2^31 - 1 rows
+ *    and serves the entry points of its own `pad` only.
  * Where host and device counts disagree the row blocks concerned are left out,
  * as in the other forms. */
-int fq_expert_plan_shape(const int64_t* host_counts, int n_experts, int64_t* shape);
+int fq_expert_plan_shape(const int64_t* host_counts, int n_experts, int pad, int64_t* shape);
 int64_t fq_expert_plan_bytes(const int64_t* shape);
 int fq_build_expert_plan(const void* counts, int counts_is_i64, int n_experts, const int64_t* shape, void* plan,
                          void* stream);
@@ -125,6 +128,13 @@ int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_i
                                  int64_t total_blocks, const void* indices, const void* probs, int probs_is_bf16,
                                  void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
                                  int64_t M, int64_t N, int round_scale, int fp8_kind, void* stream);
+
+/* fq_batched_pad_permute_quant with the tiles read from a plan of pad 16
+ * (n_experts: the width of probs). */
+int fq_batched_pad_permute_quant_planned(const void* x, const void* plan, const int64_t* shape, int n_experts,
+                                         const void* indices, const void* probs, int probs_is_bf16, void* prob_out,
+                                         void* q, float* s, void* qt, float* st, int64_t src_rows, int64_t M,
+                                         int64_t N, int round_scale, int fp8_kind, void* stream);
 
 /* triton_block_quant, linghe/quant/block.py:32-62 (kernel :11-29): one scale per
  * 128x128 block of a weight.  x bf16 [M,N], M and N multiples of 128;

@@ -31,7 +31,8 @@ SIGNATURES = {
     "fq_blockwise_quant": [_P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P],
     "fq_batched_blockwise_quant": [_P, _P, _I, _I, _L, _P, _P, _P, _P, _L, _L, _I, _I, _P],
     "fq_batched_blockwise_quant_planned": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _P],
-    "fq_expert_plan_shape": [_P, _I, _P],
+    "fq_expert_plan_shape": [_P, _I, _I, _P],
+    "fq_batched_pad_permute_quant_planned": [_P, _P, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _P],
     "fq_build_expert_plan": [_P, _I, _I, _P, _P, _P],
     "fq_batched_pad_permute_quant": [_P, _P, _I, _I, _L, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _P],
     "fq_block_quant": [_P, _P, _P, _L, _L, _I, _I, _P],

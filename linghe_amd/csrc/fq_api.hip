@@ -107,14 +107,18 @@ int fq_blockwise_quant(const void* x, void* q, float* s, void* qt, float* st, in
 
 // The per-expert entry points come in two forms that differ only in where a workgroup learns its
 // tile: from the device-side counts, or from a plan built from them (counts NULL, n_experts unused).
-static int check_plan_shape(const char* fn, const int64_t* shape, fq::PlanShape* ps) {
+static int check_plan_shape(const char* fn, const int64_t* shape, int pad, fq::PlanShape* ps) {
   FQ_REQUIRE(shape != nullptr, FQ_ERR_ARG, "%s: plan shape NULL", fn);
   FQ_REQUIRE(shape[1] >= 0 && shape[2] >= 0 && shape[3] >= 0 && shape[0] == shape[1] + shape[2] + shape[3] &&
-                 shape[0] <= (int64_t)0x3fffffff,
+                 shape[0] <= (int64_t)0x3fffffff && (shape[4] == 1 || shape[4] == 16),
              FQ_ERR_SHAPE, "%s: not a plan shape (fq_expert_plan_shape fills it)", fn);
+  // pad 0: any (the builder); otherwise the layout of the entry point that is given the plan
+  FQ_REQUIRE(pad == 0 || shape[4] == pad, FQ_ERR_SHAPE, "%s: the plan was shaped for regions padded to %lld rows, not %d",
+             fn, (long long)shape[4], pad);
   ps->unpacked = shape[1];
   ps->packed2 = shape[2];
   ps->packed4 = shape[3];
+  ps->pad = (int)shape[4];
   return FQ_OK;
 }
 
@@ -167,35 +171,37 @@ int fq_batched_blockwise_quant_planned(const void* x, const void* plan, const in
                                        void* stream) {
   const char* fn = "fq_batched_blockwise_quant_planned";
   fq::PlanShape ps;
-  int rc = check_plan_shape(fn, shape, &ps);
+  int rc = check_plan_shape(fn, shape, 1, &ps);
   if (rc) return rc;
   FQ_REQUIRE(plan != nullptr || M == 0 || shape[0] == 0, FQ_ERR_ARG, "%s: plan NULL", fn);
   return batched_blockwise_quant(fn, x, nullptr, 0, 0, plan, &ps, shape[0], q, s, qt, st, M, N, round_scale, fp8_kind,
                                  stream);
 }
 
-int fq_expert_plan_shape(const int64_t* host_counts, int n_experts, int64_t* shape) {
+int fq_expert_plan_shape(const int64_t* host_counts, int n_experts, int pad, int64_t* shape) {
   const char* fn = "fq_expert_plan_shape";
   FQ_REQUIRE(n_experts >= 0 && shape != nullptr && (host_counts != nullptr || n_experts == 0), FQ_ERR_ARG,
              "%s: NULL pointer or negative expert count", fn);
-  const fq::PlanShape ps = fq::expert_plan_shape(host_counts, n_experts);
+  FQ_REQUIRE(pad == 1 || pad == 16, FQ_ERR_ARG, "%s: pad is 1 (experts back to back) or 16", fn);
+  const fq::PlanShape ps = fq::expert_plan_shape(host_counts, n_experts, pad);
   FQ_REQUIRE(ps.blocks() <= (int64_t)0x3fffffff, FQ_ERR_SHAPE, "%s: more than 2^30 - 1 row blocks", fn);
   shape[0] = ps.blocks();
   shape[1] = ps.unpacked;
   shape[2] = ps.packed2;
   shape[3] = ps.packed4;
+  shape[4] = pad;
   return FQ_OK;
 }
 
 int64_t fq_expert_plan_bytes(const int64_t* shape) {
-  return shape == nullptr || shape[0] < 0 ? 0 : shape[0] * 16;
+  return shape == nullptr || shape[0] < 0 ? 0 : shape[0] * 20;
 }
 
 int fq_build_expert_plan(const void* counts, int counts_is_i64, int n_experts, const int64_t* shape, void* plan,
                          void* stream) {
   const char* fn = "fq_build_expert_plan";
   fq::PlanShape ps;
-  int rc = check_plan_shape(fn, shape, &ps);
+  int rc = check_plan_shape(fn, shape, 0, &ps);
   if (rc) return rc;
   FQ_REQUIRE(n_experts >= 0, FQ_ERR_SHAPE, "%s: negative expert count", fn);
   if (shape[0] == 0) return FQ_OK;
@@ -204,11 +210,13 @@ int fq_build_expert_plan(const void* counts, int counts_is_i64, int n_experts, c
                       fn);
 }
 
-int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
-                                 int64_t total_blocks, const void* indices, const void* probs, int probs_is_bf16,
-                                 void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
-                                 int64_t M, int64_t N, int round_scale, int fp8_kind, void* stream) {
-  const char* fn = "fq_batched_pad_permute_quant";
+}  // extern "C"
+
+static int batched_pad_permute_quant(const char* fn, const void* x, const void* counts, int counts_is_i64,
+                                     int n_experts, const void* plan, const fq::PlanShape* ps, int64_t total_blocks,
+                                     const void* indices, const void* probs, int probs_is_bf16, void* prob_out,
+                                     void* q, float* s, void* qt, float* st, int64_t src_rows, int64_t M, int64_t N,
+                                     int round_scale, int fp8_kind, void* stream) {
   int rc = check_common(fn, M, N, round_scale, fp8_kind);
   if (rc) return rc;
   if (M == 0) return FQ_OK;  // nothing routed: there is nothing to write (and empty outputs may be NULL)
@@ -219,14 +227,38 @@ int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_i
   if ((rc = check_mode_ptrs(fn, 2, q, s, qt, st))) return rc;
   FQ_REQUIRE((probs == nullptr) == (prob_out == nullptr), FQ_ERR_ARG, "%s: probs and prob_out go together", fn);
   if (M == 0 || total_blocks == 0 || src_rows == 0) return FQ_OK;
-  FQ_REQUIRE(x && aligned16(x) && counts && indices && aligned16(indices), FQ_ERR_ARG,
-             "%s: x/counts/indices NULL or misaligned", fn);
-  FQ_REQUIRE(total_blocks <= (M + 127) / 128 + n_experts, FQ_ERR_SHAPE, "%s: total_blocks inconsistent with M", fn);
+  FQ_REQUIRE(x && aligned16(x) && indices && aligned16(indices), FQ_ERR_ARG, "%s: x/indices NULL or misaligned", fn);
+  if ((rc = check_batch_source(fn, counts, n_experts, plan, total_blocks, M))) return rc;
   if ((rc = check_tiles(fn, total_blocks * (N / 128)))) return rc;
   return check_launch(fq::launch_pad_permute_quant(x, indices, probs, probs_is_bf16 != 0, prob_out, q, s, qt, st,
                                                    src_rows, M, (int)N, round_scale, fp8_kind, counts,
-                                                   counts_is_i64 != 0, n_experts, total_blocks, (hipStream_t)stream),
+                                                   counts_is_i64 != 0, n_experts, total_blocks, (hipStream_t)stream,
+                                                   plan, ps),
                       fn);
+}
+
+extern "C" {
+
+int fq_batched_pad_permute_quant(const void* x, const void* counts, int counts_is_i64, int n_experts,
+                                 int64_t total_blocks, const void* indices, const void* probs, int probs_is_bf16,
+                                 void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
+                                 int64_t M, int64_t N, int round_scale, int fp8_kind, void* stream) {
+  return batched_pad_permute_quant("fq_batched_pad_permute_quant", x, counts, counts_is_i64, n_experts, nullptr,
+                                   nullptr, total_blocks, indices, probs, probs_is_bf16, prob_out, q, s, qt, st,
+                                   src_rows, M, N, round_scale, fp8_kind, stream);
+}
+
+int fq_batched_pad_permute_quant_planned(const void* x, const void* plan, const int64_t* shape, int n_experts,
+                                         const void* indices, const void* probs, int probs_is_bf16, void* prob_out,
+                                         void* q, float* s, void* qt, float* st, int64_t src_rows, int64_t M,
+                                         int64_t N, int round_scale, int fp8_kind, void* stream) {
+  const char* fn = "fq_batched_pad_permute_quant_planned";
+  fq::PlanShape ps;
+  int rc = check_plan_shape(fn, shape, 16, &ps);
+  if (rc) return rc;
+  FQ_REQUIRE(plan != nullptr || M == 0 || shape[0] == 0, FQ_ERR_ARG, "%s: plan NULL", fn);
+  return batched_pad_permute_quant(fn, x, nullptr, 0, n_experts, plan, &ps, shape[0], indices, probs, probs_is_bf16,
+                                   prob_out, q, s, qt, st, src_rows, M, N, round_scale, fp8_kind, stream);
 }
 
 int fq_group_quant(const void* x, void* q, float* s, int64_t M, int64_t N, int round_scale, int fp8_kind,
@@ -522,7 +554,7 @@ int fq_batched_swiglu_quant_fwd_planned(const void* x, const void* weight, int w
                                         int64_t n, int round_scale, int output_mode, int fp8_kind, void* stream) {
   const char* fn = "fq_batched_swiglu_quant_fwd_planned";
   fq::PlanShape ps;
-  int rc = check_plan_shape(fn, shape, &ps);
+  int rc = check_plan_shape(fn, shape, 1, &ps);
   if (rc) return rc;
   FQ_REQUIRE(plan != nullptr || M == 0 || shape[0] == 0, FQ_ERR_ARG, "%s: plan NULL", fn);
   return batched_swiglu_quant_fwd(fn, x, weight, weight_is_bf16, nullptr, 0, 0, plan, &ps, shape[0], q, s, qt, st, M,
@@ -544,7 +576,7 @@ int fq_batched_swiglu_quant_bwd_planned(const void* g, const void* x, const void
                                         int round_scale, int fp8_kind, void* stream) {
   const char* fn = "fq_batched_swiglu_quant_bwd_planned";
   fq::PlanShape ps;
-  int rc = check_plan_shape(fn, shape, &ps);
+  int rc = check_plan_shape(fn, shape, 1, &ps);
   if (rc) return rc;
   FQ_REQUIRE(plan != nullptr || M == 0 || shape[0] == 0, FQ_ERR_ARG, "%s: plan NULL", fn);
   return batched_swiglu_quant_bwd(fn, g, x, weight, weight_is_bf16, nullptr, 0, 0, plan, &ps, shape[0], dq, ds, dw, dqt,

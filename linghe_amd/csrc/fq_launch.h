@@ -11,6 +11,7 @@ namespace fq {
 // of 33..64 rows, last blocks of at most 32 rows (counted on the host from its copy of the counts)
 struct PlanShape {
   int64_t unpacked, packed2, packed4;
+  int pad;  // 1: experts back to back; 16: every expert's region of the outputs rounded up to 16 rows
   int64_t blocks() const { return unpacked + packed2 + packed4; }
 };
 
@@ -22,7 +23,8 @@ hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, fl
 hipError_t launch_pad_permute_quant(const void* x, const void* indices, const void* probs, int probs_bf16,
                                     void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
                                     int64_t M, int N, int round_scale, int kind, const void* counts, int counts_i64,
-                                    int n_experts, int64_t row_blocks, hipStream_t stream);
+                                    int n_experts, int64_t row_blocks, hipStream_t stream, const void* plan = nullptr,
+                                    const PlanShape* ps = nullptr);
 
 hipError_t launch_silu_quant_fwd(const void* x, const void* weight, int weight_bf16, void* q, float* s, void* qt,
                                  float* st, int64_t M, int n, int round_scale, int mode, int kind,
@@ -38,7 +40,7 @@ hipError_t launch_silu_quant_bwd(const void* g, const void* x, const void* weigh
 // Per-expert launches with `plan` (expert_plan_bytes(ps) bytes of device memory filled by
 // launch_expert_plan from the same counts) and its shape read their tile from it instead of
 // scanning the counts; counts may then be NULL and row_blocks is not used.
-PlanShape expert_plan_shape(const int64_t* host_counts, int n_experts);
+PlanShape expert_plan_shape(const int64_t* host_counts, int n_experts, int pad);
 int64_t expert_plan_bytes(const PlanShape& ps);
 hipError_t launch_expert_plan(const void* counts, int counts_i64, int n_experts, const PlanShape& ps, void* plan,
                               hipStream_t stream);

@@ -82,6 +82,7 @@ struct Policy {
   static constexpr bool kPlanPackedFirstSiluFwd = false;
   static constexpr bool kPlanPackedFirstSiluBwd = false;
   static constexpr bool kPlanPackedFirstBlockwise = true;
+  static constexpr bool kPlanPackedFirstPermute = false;  // 43.8 / 43.3 us first / last (33040 x 2048 gathered from 16384 rows)
   // row blocks per run that an XCD works on (xcd_runs; 0: every eighth tile).  Same sizes, planned launches with
   // 0 / 2 / 4 / 8 / 16: SwiGLU forward 43.4 / 41.2 / 40.8 / 40.7 / 40.8 us, backward 76.5 / 76.1 / 75.5 / 75.3 / 76.2,
   // blockwise quantiser 30.9 / 30.3 / 29.9 / 29.9 / 29.8.  Launches that scan the counts, 0 / 2 / 4 / 8: forward
@@ -89,6 +90,11 @@ struct Policy {
   // gather + pad + quant 47.0 / 48.8 / 49.4 / 50.8: only the backward gains there
   static constexpr int kXcdRowsPlanned = 8;
   static constexpr int kXcdRowsSiluBwdCounts = 4;
+  // gather + pad + quant with a plan: runs of 8 row blocks per XCD 50.6 us, grid order 44.8, column sweeps (-1:
+  // XCD X takes the column blocks X, X + 8, .. one after the other, so that what it gathers from while it works
+  // on one of them is a 256-byte strip of the source: 4.2 MB for 16384 source rows, the size of its L2) 43.8;
+  // the launch that scans the counts 45.6
+  static constexpr int kXcdRowsPermutePlanned = -1;
   static constexpr bool kStartPriorityRmsnorm = true;
   // RMSNorm + quant in two passes, both passes giving XCD X (workgroup number mod 8) the X-th eighth of the rows,
   // the statistic pass walking its eighth from the end and the tile kernel from the start: what the tile kernel

@@ -38,8 +38,7 @@ struct BatchArgs {
 // What a workgroup of a per-expert launch needs to know about its 128-row block, written once per
 // set of counts by expert_plan_kernel and read with one 16-byte load through the constant path
 // instead of the prefix scan over all counts (which puts a dependent vector load and three wave
-// scans in front of every workgroup's first tile load).  Experts lie back to back (no padding of
-// their regions).  Three sections, each in expert order: the row blocks that are worked on
+// scans in front of every workgroup's first tile load).  Three sections, each in expert order: the row blocks that are worked on
 // unpacked (all but an expert's last one, and last ones of more than 64 rows), the last blocks of
 // 33..64 rows (two column blocks to a workgroup), the last blocks of at most 32 rows (four).  The
 // host knows the sizes of the sections from its copy of the counts, sizes the launch for exactly
@@ -48,11 +47,13 @@ struct BatchArgs {
 // Records are small because they are read cold: every line of the table that a workgroup is the
 // first of its XCD to touch costs it a trip to memory before its first tile load can leave.
 struct PlanEntry {
-  uint32_t row0;   // first global row of the row block
+  uint32_t row0;   // first global row of the row block (in the outputs: regions padded when BatchArgs::pad says so)
   int rb;          // row block inside the expert
   int count;       // rows of the expert
   uint32_t where;  // kind << 30 | row block in expert order over all experts (row of the transposed scales)
 };
+// behind the records: one int per record, the expert it belongs to (read only by the kernel that
+// needs it, gather + pad + quant for its probabilities)
 constexpr uint32_t kPlanEmpty = 0, kPlanUnpacked = 1, kPlanPacked2 = 2, kPlanPacked4 = 3;  // kinds
 static_assert(sizeof(PlanEntry) == 16, "16-byte records");
 
@@ -143,26 +144,39 @@ __device__ __forceinline__ TileGeom resolve_tile(int64_t M, int ncb, int64_t out
       if (b.xcd_rows > 0) r = xcd_runs(r, b.plan_unpacked * ncb, b.xcd_rows * ncb);
       idx = r / ncb;
       x = r - idx * ncb;
+      if (b.xcd_rows < 0 && (ncb & 7) == 0) {
+        // column sweeps: XCD X takes the column blocks X, X + 8, ... one after the other, each over all row
+        // blocks (what an XCD reads while it works on one column block is a 256-byte-wide strip of the source)
+        const int xcd = r & 7, pos = r >> 3;
+        const int cbi = pos / b.plan_unpacked;
+        idx = pos - cbi * b.plan_unpacked;
+        x = xcd + 8 * cbi;
+      }
     }
+    const int n_records = b.plan_unpacked + b.plan_packed2 + b.plan_packed4;
     const_u32 e = (const_u32)((uintptr_t)b.plan + (uintptr_t)idx * sizeof(PlanEntry));
     const uint32_t row0 = e[0], where = e[3];
     const int rb = (int)e[1], count = (int)e[2];
+    g.expert = 0;
+    if (b.pad > 1)  // the one kernel that pads is the one that asks for the expert
+      g.expert = (int)((const_u32)((uintptr_t)b.plan + (uintptr_t)n_records * sizeof(PlanEntry)))[idx];
     g.kc_shift = (int)kind - 1;
+    const int pcount = b.pad > 1 ? (count + b.pad - 1) & -b.pad : count;
     const int64_t row_start = (int64_t)row0 - (int64_t)rb * kGroup;
     const int left = count - rb * kGroup;
+    const int pleft = pcount - rb * kGroup;
     g.cb = x << g.kc_shift;
     const int cbs_left = ncb - g.cb;
     g.n_sub = cbs_left < (1 << g.kc_shift) ? cbs_left : (1 << g.kc_shift);
     // a record of another kind than its section's: the host's counts are not the device's
-    g.valid = (where >> 30) == kind && idx < b.plan_unpacked + b.plan_packed2 + b.plan_packed4;
-    g.expert = 0;  // not recorded: no kernel that takes a plan asks for it
+    g.valid = (where >> 30) == kind && idx < n_records;
     g.rows_valid = left < kGroup ? left : kGroup;
-    g.rows_store = g.rows_valid;
+    g.rows_store = pleft < kGroup ? pleft : kGroup;
     g.row0 = (int64_t)row0;
     g.s_base = row_start * (out_w / kGroup) + (int64_t)rb * kGroup;
-    g.s_stride = count;
+    g.s_stride = pcount;
     g.t_base = row_start * out_w + (int64_t)rb * kGroup;
-    g.t_stride = count;
+    g.t_stride = pcount;
     g.st_row = (int64_t)(where & 0x3fffffffu);
     if (g.row0 + g.rows_store > M) g.valid = false;
   } else {

@@ -348,8 +348,9 @@ __global__ __launch_bounds__(2048 / Policy::kRowsPerThreadRmsnorm) void rmsnorm_
 // surplus is dropped (the launches then leave those row blocks out: the counts disagree).
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restrict__ counts, int counts_i64,
-                                                           int n_experts, int b0, int b1, int b2,
+                                                           int n_experts, int pad, int b0, int b1, int b2,
                                                            PlanEntry* __restrict__ plan) {
+  int* __restrict__ expert_of = (int*)(plan + ((int64_t)b0 + b1 + b2));
   constexpr int T = 1024, W = T / 64;
   __shared__ int eb[T + 1];  // exclusive sums of the pass: row blocks,
   __shared__ int ez[T];      // unpacked row blocks,
@@ -366,8 +367,9 @@ __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restric
     const int e = base + t;
     const int cr = e < n_experts ? load_count(counts, counts_i64, e) : 0;
     const int c = cr > 0 ? cr : 0;
+    const int pc = (c + pad - 1) & -pad;  // rows of the expert's region in the outputs (pad: 1 or 16)
     const int nb = (c + kGroup - 1) / kGroup;
-    const int sh = nb > 0 ? pack_shift(c - (nb - 1) * kGroup) : 0;
+    const int sh = nb > 0 ? pack_shift(pc - (nb - 1) * kGroup) : 0;
     const int p = (sh == 1) + ((sh == 2) << 16);
     const int z = nb - (sh > 0);
     const int ib = wave_inclusive_scan(nb);
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restric
     const int ip = wave_inclusive_scan(p);
     // the rows of 64 experts fit 32 bits for every matrix the entry points accept; the sums over
     // waves and passes are 64-bit
-    const int ir = wave_inclusive_scan(c);
+    const int ir = wave_inclusive_scan(pc);
     if (lane == 63) { wb[wave] = ib; wz[wave] = iz; wp[wave] = ip; wr[wave] = ir; }
     __syncthreads();
     int ob = 0, oz = 0, op = 0;
@@ -384,7 +386,7 @@ __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restric
     eb[t] = ob + ib - nb;
     ez[t] = oz + iz - z;
     ep[t] = op + ip - p;
-    er[t] = orow + ir - c;
+    er[t] = orow + ir - pc;
     ec[t] = c;
     if (t == T - 1) {
       eb[T] = ob + ib;
@@ -401,7 +403,7 @@ __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restric
       }
       const int cl = ec[lo], rb = j - eb[lo];
       const int nbl = (cl + kGroup - 1) / kGroup;
-      const int shift = rb == nbl - 1 ? pack_shift(cl - rb * kGroup) : 0;
+      const int shift = rb == nbl - 1 ? pack_shift(((cl + pad - 1) & -pad) - rb * kGroup) : 0;
       // place inside the record's section, the section's start and size
       const int64_t in = shift == 0 ? (int64_t)run_z + ez[lo] + rb
                          : shift == 1 ? (int64_t)run_p1 + (ep[lo] & 0xffff) : (int64_t)run_p2 + (ep[lo] >> 16);
@@ -415,10 +417,11 @@ __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restric
         pe.where = (shift == 0 ? kPlanUnpacked : shift == 1 ? kPlanPacked2 : kPlanPacked4) << 30 |
                    (uint32_t)(run_blocks + j);
         plan[first + in] = pe;
+        expert_of[first + in] = base + lo;
       }
     }
     run_blocks += pass_blocks;
-    run_rows += er[T - 1] + ec[T - 1];
+    run_rows += er[T - 1] + ((ec[T - 1] + pad - 1) & -pad);
     run_z += pass_z;
     run_p1 += pass_p & 0xffff;
     run_p2 += pass_p >> 16;
@@ -429,31 +432,32 @@ __global__ __launch_bounds__(1024) void expert_plan_kernel(const void* __restric
   none.rb = 0;
   none.count = 0;
   none.where = kPlanEmpty << 30;
-  for (int64_t at = (int64_t)run_z + t; at < b0; at += T) plan[at] = none;
-  for (int64_t at = (int64_t)b0 + run_p1 + t; at < (int64_t)b0 + b1; at += T) plan[at] = none;
-  for (int64_t at = (int64_t)b0 + b1 + run_p2 + t; at < (int64_t)b0 + b1 + b2; at += T) plan[at] = none;
+  for (int64_t at = (int64_t)run_z + t; at < b0; at += T) { plan[at] = none; expert_of[at] = -1; }
+  for (int64_t at = (int64_t)b0 + run_p1 + t; at < (int64_t)b0 + b1; at += T) { plan[at] = none; expert_of[at] = -1; }
+  for (int64_t at = (int64_t)b0 + b1 + run_p2 + t; at < (int64_t)b0 + b1 + b2; at += T) { plan[at] = none; expert_of[at] = -1; }
 }
 
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
 static BatchArgs batch_args(const void* counts, int counts_i64, int n_experts, const void* plan,
-                            const PlanShape* ps, bool packed_first, int xcd_rows_scan) {
+                            const PlanShape* ps, bool packed_first, int xcd_rows_scan,
+                            int xcd_rows_planned = Policy::kXcdRowsPlanned) {
   if (plan != nullptr)
-    return BatchArgs{nullptr, 0, 0, 0, plan, (int)ps->unpacked, (int)ps->packed2, (int)ps->packed4,
-                     Policy::kXcdRowsPlanned, packed_first};
+    return BatchArgs{nullptr, 0, n_experts, ps->pad > 1 ? ps->pad : 0, plan, (int)ps->unpacked, (int)ps->packed2,
+                     (int)ps->packed4, xcd_rows_planned, packed_first};
   return BatchArgs{counts, counts_i64, n_experts, 0, nullptr, 0, 0, 0, xcd_rows_scan, 0};
 }
 
-int64_t expert_plan_bytes(const PlanShape& ps) { return ps.blocks() * (int64_t)sizeof(PlanEntry); }
+int64_t expert_plan_bytes(const PlanShape& ps) { return ps.blocks() * (int64_t)(sizeof(PlanEntry) + sizeof(int)); }
 
-PlanShape expert_plan_shape(const int64_t* host_counts, int n_experts) {
-  PlanShape ps{0, 0, 0};
+PlanShape expert_plan_shape(const int64_t* host_counts, int n_experts, int pad) {
+  PlanShape ps{0, 0, 0, pad};
   for (int e = 0; e < n_experts; ++e) {
     const int64_t c = host_counts[e] > 0 ? host_counts[e] : 0;
     const int64_t nb = (c + kGroup - 1) / kGroup;
     if (nb == 0) continue;
-    const int last = (int)(c - (nb - 1) * kGroup);
+    const int last = (int)(((c + pad - 1) & -(int64_t)pad) - (nb - 1) * kGroup);
     const int shift = last <= 32 ? 2 : last <= 64 ? 1 : 0;  // pack_shift, on the host
     ps.unpacked += nb - (shift > 0);
     ps.packed2 += shift == 1;
@@ -465,7 +469,7 @@ PlanShape expert_plan_shape(const int64_t* host_counts, int n_experts) {
 hipError_t launch_expert_plan(const void* counts, int counts_i64, int n_experts, const PlanShape& ps, void* plan,
                               hipStream_t stream) {
   if (ps.blocks() == 0) return hipSuccess;
-  hipLaunchKernelGGL(expert_plan_kernel, dim3(1), dim3(1024), 0, stream, counts, counts_i64, n_experts,
+  hipLaunchKernelGGL(expert_plan_kernel, dim3(1), dim3(1024), 0, stream, counts, counts_i64, n_experts, ps.pad,
                      (int)ps.unpacked, (int)ps.packed2, (int)ps.packed4, (PlanEntry*)plan);
   return hipGetLastError();
 }
@@ -495,10 +499,14 @@ hipError_t launch_blockwise_quant(const void* x, void* q, float* s, void* qt, fl
 hipError_t launch_pad_permute_quant(const void* x, const void* indices, const void* probs, int probs_bf16,
                                     void* prob_out, void* q, float* s, void* qt, float* st, int64_t src_rows,
                                     int64_t M, int N, int round_scale, int kind, const void* counts, int counts_i64,
-                                    int n_experts, int64_t row_blocks, hipStream_t stream) {
+                                    int n_experts, int64_t row_blocks, hipStream_t stream, const void* plan,
+                                    const PlanShape* ps) {
   OutPtrs out{(uint8_t*)q, s, (uint8_t*)qt, st};
   BatchArgs b{counts, counts_i64, n_experts, 16, nullptr, 0, 0, 0, 0, 0};
-  const int64_t tiles = row_blocks * (N / kGroup);
+  if (plan != nullptr)
+    b = batch_args(nullptr, 0, n_experts, plan, ps, Policy::kPlanPackedFirstPermute, 0, Policy::kXcdRowsPermutePlanned);
+  const int64_t tiles = plan ? plan_workgroups(ps->unpacked, ps->packed2, ps->packed4, N / kGroup)
+                             : row_blocks * (N / kGroup);
   if (tiles == 0) return hipSuccess;
   const dim3 grid((unsigned)tiles), block(256);
   FQ_DISPATCH_KIND(kind, K,

@@ -92,7 +92,7 @@ def triton_batch_blockwise_quant(xs, token_count_per_expert, splits, round_scale
     if M == 0:
         return x_q, x_scale, xt_q, xt_scale
     if plan is not None:
-        if plan.blocks != blocks or plan.table.device != device:
+        if plan.blocks != blocks or plan.pad != 1 or plan.table.device != device:
             raise ValueError("plan does not belong to these splits / this device")
         with _lib.on_device(device):
             _lib.check(_lib.lib.fq_batched_blockwise_quant_planned(

@@ -12,7 +12,7 @@ from .. import _lib
 
 def triton_batch_block_pad_permute_with_indices(
     xs, token_count_per_expert, indices, splits, probs=None, round_scale=False, *,
-    fp8_dtype=torch.float8_e4m3fn
+    fp8_dtype=torch.float8_e4m3fn, plan=None
 ):
     """
     select and quant, used in megatron 0.12 flex moe
@@ -24,6 +24,7 @@ def triton_batch_block_pad_permute_with_indices(
         splits: python int list of token_count_per_expert
         probs: route weights, [bs, n_experts]
         round_scale: whether round scale to power of 2
+        plan: optional linghe_amd.utils.silu.ExpertPlan of the same counts built with pad=16
 
     Returns:
         x_q [M, dim], x_scale [M, dim/128] (per expert [dim/128, padded count]),
@@ -66,6 +67,15 @@ def triton_batch_block_pad_permute_with_indices(
             pbf16 = 1
         elif probs.dtype != torch.float32:
             raise TypeError(f"probs must be float32 or bfloat16, got {probs.dtype}")
+    if plan is not None:
+        if plan.blocks != blocks or plan.pad != 16 or plan.table.device != device:
+            raise ValueError("plan does not belong to these splits / this layout (pad=16) / this device")
+        with _lib.on_device(device):
+            _lib.check(_lib.lib.fq_batched_pad_permute_quant_planned(
+                _lib.ptr(xs), _lib.ptr(plan.table), plan.shape, n_experts, _lib.ptr(indices), _lib.ptr(probs), pbf16,
+                _lib.ptr(prob_output), _lib.ptr(x_q), _lib.ptr(x_scale), _lib.ptr(xt_q), _lib.ptr(xt_scale), m, M, N,
+                int(bool(round_scale)), _lib.fp8_kind(fp8_dtype), _lib.stream_of(xs)))
+        return x_q, x_scale, xt_q, xt_scale, prob_output
     with _lib.on_device(device):
         _lib.check(_lib.lib.fq_batched_pad_permute_quant(
             _lib.ptr(xs), _lib.ptr(counts), is64, n_experts, blocks, _lib.ptr(indices),

@@ -26,22 +26,25 @@ class ExpertPlan:
     ``splits`` instead.
     """
 
-    __slots__ = ("table", "shape", "blocks")
+    __slots__ = ("table", "shape", "blocks", "pad")
 
     def __init__(self, table: torch.Tensor, shape):
         self.table = table
-        self.shape = shape            # ctypes int64[4]: row blocks, whole / halved / quartered ones
+        self.shape = shape            # ctypes int64[5]: row blocks, whole / halved / quartered ones, pad
         self.blocks = int(shape[0])
+        self.pad = int(shape[4])
 
 
-def build_expert_plan(counts: torch.Tensor, splits) -> ExpertPlan:
-    """counts: device int32/int64 [n_experts]; splits: the same numbers as a python list."""
+def build_expert_plan(counts: torch.Tensor, splits, pad: int = 1) -> ExpertPlan:
+    """counts: device int32/int64 [n_experts]; splits: the same numbers as a python list;
+    pad: 1 for the layouts with the experts back to back (SwiGLU, blockwise quantiser), 16 for
+    gather + pad + quant (every expert's region of the outputs rounded up to 16 rows)."""
     import ctypes
 
     n = len(splits)
     host = (ctypes.c_int64 * max(n, 1))(*[int(c) for c in splits])
-    shape = (ctypes.c_int64 * 4)()
-    _lib.check(_lib.lib.fq_expert_plan_shape(host, n, shape))
+    shape = (ctypes.c_int64 * 5)()
+    _lib.check(_lib.lib.fq_expert_plan_shape(host, n, pad, shape))
     nbytes = int(_lib.lib.fq_expert_plan_bytes(shape))
     table = torch.empty((max(nbytes, 16),), device=counts.device, dtype=torch.uint8)
     if shape[0]:
@@ -55,6 +58,8 @@ def build_expert_plan(counts: torch.Tensor, splits) -> ExpertPlan:
 def _check_plan(plan: ExpertPlan, blocks: int, device) -> None:
     if plan.blocks != blocks:
         raise ValueError(f"plan was built for {plan.blocks} row blocks, splits give {blocks}")
+    if plan.pad != 1:
+        raise ValueError("plan was built for the padded layout of gather + pad + quant")
     if plan.table.device != device:
         raise ValueError("plan lives on another device")
 

@@ -255,17 +255,23 @@ def test_expert_plan_shape_on_host():
     }
     for counts, want in cases.items():
         host = (ctypes.c_int64 * max(len(counts), 1))(*counts)
-        shape = (ctypes.c_int64 * 4)(-1, -1, -1, -1)
-        assert L.fq_expert_plan_shape(host, len(counts), shape) == 0
-        assert list(shape) == want, (counts, list(shape))
-        assert L.fq_expert_plan_bytes(shape) == 16 * want[0]
-    assert L.fq_expert_plan_shape(None, 3, shape) == -1
-    bad = (ctypes.c_int64 * 4)(5, 1, 1, 1)  # the parts do not add up
+        shape = (ctypes.c_int64 * 5)(-1, -1, -1, -1, -1)
+        assert L.fq_expert_plan_shape(host, len(counts), 1, shape) == 0
+        assert list(shape) == want + [1], (counts, list(shape))
+        assert L.fq_expert_plan_bytes(shape) == 20 * want[0]
+    # the padded layout of gather + pad + quant classes a last block by its rows rounded up to 16
+    host = (ctypes.c_int64 * 4)(32, 33, 64, 65)
+    assert L.fq_expert_plan_shape(host, 4, 16, shape) == 0 and list(shape) == [4, 1, 2, 1, 16]
+    host = (ctypes.c_int64 * 3)(17, 49, 129)   # 32 | 64 | 128 + 16
+    assert L.fq_expert_plan_shape(host, 3, 16, shape) == 0 and list(shape) == [4, 1, 1, 2, 16]
+    assert L.fq_expert_plan_shape(host, 3, 8, shape) == -1
+    assert L.fq_expert_plan_shape(None, 3, 1, shape) == -1
+    bad = (ctypes.c_int64 * 5)(5, 1, 1, 1, 1)  # the parts do not add up
     rc = L.fq_batched_blockwise_quant_planned(None, ctypes.c_void_p(256), bad, None, None, None, None, 640, 128, 0, 0,
                                               None)
     assert rc == -2 and b"plan shape" in L.fq_last_error()
     assert L.fq_build_expert_plan(None, 0, 4, bad, ctypes.c_void_p(256), None) == -2
-    good = (ctypes.c_int64 * 4)(3, 1, 1, 1)
+    good = (ctypes.c_int64 * 5)(3, 1, 1, 1, 1)
     # more row blocks than rows
     rc = L.fq_batched_swiglu_quant_fwd_planned(ctypes.c_void_p(256), ctypes.c_void_p(256), 0, ctypes.c_void_p(256),
                                                good, ctypes.c_void_p(256), ctypes.c_void_p(256), ctypes.c_void_p(256),
@@ -277,3 +283,7 @@ def test_expert_plan_shape_on_host():
                                                ctypes.c_void_p(256), ctypes.c_void_p(256), ctypes.c_void_p(256),
                                                ctypes.c_void_p(256), 640, 128, 0, 0, None)
     assert rc == -1 and b"plan NULL" in L.fq_last_error()
+    # a plan of the back-to-back layout handed to gather + pad + quant
+    rc = L.fq_batched_pad_permute_quant_planned(None, ctypes.c_void_p(256), good, 4, None, None, 0, None, None, None,
+                                                None, None, 64, 64, 256, 0, 0, None)
+    assert rc == -2 and b"padded" in L.fq_last_error()

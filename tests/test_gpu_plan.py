@@ -21,31 +21,41 @@ def _kind(rows):
     return 3 if rows <= 32 else 2 if rows <= 64 else 1
 
 
-def _expected_shape(counts):
-    """row blocks in all, worked on whole (kind 1), in halves (2: a last block of 33..64 rows), in quarters (3)"""
-    kinds = [_kind(min(128, c - rb * 128)) for c in counts for rb in range((c + 127) // 128)]
-    return [len(kinds)] + [kinds.count(k) for k in (1, 2, 3)]
+def _blocks(counts, pad):
+    """(first row in the outputs, row block inside the expert, count, kind, expert) of every row block, expert order"""
+    out, start = [], 0
+    for e, c in enumerate(counts):
+        pc = (c + pad - 1) // pad * pad
+        for rb in range((c + 127) // 128):
+            out.append((start + rb * 128, rb, c, _kind(min(128, pc - rb * 128)), e))
+        start += pc
+    return out
+
+
+def _expected_shape(counts, pad=1):
+    """row blocks in all, worked on whole (kind 1), in halves (2: a last block whose padded rows are 33..64), in
+    quarters (3), and the padding itself"""
+    kinds = [b[3] for b in _blocks(counts, pad)]
+    return [len(kinds)] + [kinds.count(k) for k in (1, 2, 3)] + [pad]
 
 
 def _expected_plan(counts, shape):
-    """[blocks, 4] uint32 records: a row block's first row, its number inside the expert, the
-    expert's count, and kind << 30 | its number over all experts; three sections (kinds 1, 2, 3)
-    of the sizes in `shape`, each in expert order, what the counts do not fill left zero and what
-    they have beyond a section's size dropped."""
+    """[blocks, 4] uint32 records - a row block's first row, its number inside the expert, the expert's
+    count, kind << 30 | its number over all experts - and [blocks] int32 experts behind them; three sections
+    (kinds 1, 2, 3) of the sizes in `shape`, each in expert order, what the counts do not fill left zero
+    (expert -1) and what they have beyond a section's size dropped."""
     first = [0, shape[1], shape[1] + shape[2]]
-    size = shape[1:]
+    size = shape[1:4]
     fill = [0, 0, 0]
     table = np.zeros((shape[0], 4), dtype=np.int64)
-    start = rbg = 0
-    for c in counts:
-        for rb in range((c + 127) // 128):
-            k = _kind(min(128, c - rb * 128)) - 1
-            if fill[k] < size[k]:
-                table[first[k] + fill[k]] = [start + rb * 128, rb, c, (k + 1) << 30 | rbg]
-            fill[k] += 1
-            rbg += 1
-        start += c
-    return table.astype(np.uint32)
+    experts = np.full((shape[0],), -1, dtype=np.int32)
+    for rbg, (row0, rb, c, kind, e) in enumerate(_blocks(counts, shape[4])):
+        k = kind - 1
+        if fill[k] < size[k]:
+            table[first[k] + fill[k]] = [row0, rb, c, kind << 30 | rbg]
+            experts[first[k] + fill[k]] = e
+        fill[k] += 1
+    return table.astype(np.uint32), experts
 
 
 COUNT_SETS = {
@@ -65,34 +75,36 @@ def _many_experts():
 
 
 @pytest.mark.parametrize("name", sorted(COUNT_SETS) + ["many"])
-@pytest.mark.parametrize("cdt", [torch.int32, torch.int64])
-def test_plan_records(gpu, name, cdt):
+@pytest.mark.parametrize("cdt,pad", [(torch.int32, 1), (torch.int64, 1), (torch.int32, 16)])
+def test_plan_records(gpu, name, cdt, pad):
     import ctypes
 
     from linghe_amd import _lib
 
     counts = _many_experts() if name == "many" else COUNT_SETS[name]
-    announce("expert plan records", name, cdt)
+    announce("expert plan records", name, cdt, pad)
     host = (ctypes.c_int64 * len(counts))(*counts)
-    shape = (ctypes.c_int64 * 4)()
-    _lib.check(_lib.lib.fq_expert_plan_shape(host, len(counts), shape))
-    assert list(shape) == _expected_shape(counts)
+    shape = (ctypes.c_int64 * 5)()
+    _lib.check(_lib.lib.fq_expert_plan_shape(host, len(counts), pad, shape))
+    assert list(shape) == _expected_shape(counts, pad)
     cnt = torch.tensor(counts, dtype=cdt, device=gpu)
     # the host's shape may disagree with the device's counts: sections are never overrun, their rest is empty
     for delta in ((0, 0, 0), (2, 1, 3), (-1, -1, -1)):
         sh = [max(0, shape[1 + i] + delta[i]) for i in range(3)]
-        sh = [sum(sh)] + sh
+        sh = [sum(sh)] + sh + [pad]
         if sh[0] == 0:
             continue
-        cs = (ctypes.c_int64 * 4)(*sh)
+        cs = (ctypes.c_int64 * 5)(*sh)
         nbytes = int(_lib.lib.fq_expert_plan_bytes(cs))
-        assert nbytes == 16 * sh[0]
+        assert nbytes == 20 * sh[0]
         table = torch.full((nbytes,), 0x5A, dtype=torch.uint8, device=gpu)
         _lib.check(_lib.lib.fq_build_expert_plan(_lib.ptr(cnt), int(cdt == torch.int64), len(counts), cs,
                                                  _lib.ptr(table), _lib.stream_of(cnt)))
         torch.cuda.synchronize()
-        got = table.cpu().numpy().view(np.uint32).reshape(sh[0], 4)
-        np.testing.assert_array_equal(got, _expected_plan(counts, sh))
+        raw = table.cpu().numpy()
+        records, experts = _expected_plan(counts, sh)
+        np.testing.assert_array_equal(raw[:16 * sh[0]].view(np.uint32).reshape(sh[0], 4), records)
+        np.testing.assert_array_equal(raw[16 * sh[0]:].view(np.int32), experts)
 
 
 @pytest.mark.parametrize("name", sorted(COUNT_SETS) + ["many"])
@@ -190,7 +202,7 @@ def test_planned_launch_with_larger_shape_than_the_counts(gpu):
     ref = triton_batch_blockwise_quant(x, cnt, counts)
     exact = _expected_shape(counts)
     sh = [exact[1] + 2, exact[2] + 1, exact[3] + 3]
-    shape = (ctypes.c_int64 * 4)(sum(sh), *sh)
+    shape = (ctypes.c_int64 * 5)(sum(sh), *sh, 1)
     table = torch.empty((int(_lib.lib.fq_expert_plan_bytes(shape)),), dtype=torch.uint8, device=gpu)
     L = _lib.lib
     _lib.check(L.fq_build_expert_plan(_lib.ptr(cnt), 0, len(counts), shape, _lib.ptr(table), _lib.stream_of(x)))
@@ -201,3 +213,35 @@ def test_planned_launch_with_larger_shape_than_the_counts(gpu):
     torch.cuda.synchronize()
     for u, v in zip(ref, out):
         assert torch.equal(u.view(torch.uint8), v.view(torch.uint8))
+
+
+@pytest.mark.parametrize("name", ["mixed", "ragged", "zipf300", "one"])
+@pytest.mark.parametrize("with_probs", [True, False])
+def test_planned_pad_permute_quant(gpu, name, with_probs):
+    """gather + pad + quant with a plan of the padded layout: every output (the gathered
+    probabilities included, which need the expert of a tile) byte for byte."""
+    from linghe_amd.utils.gather import triton_batch_block_pad_permute_with_indices as permute
+    from linghe_amd.utils.silu import build_expert_plan
+
+    counts = COUNT_SETS[name]
+    announce("planned gather + pad + quant", name, with_probs)
+    g = gen(36)
+    m, N = 700, 384
+    x = _dev(randn_bf16(g, m, N), gpu)
+    probs = _dev(torch.rand(m, len(counts), generator=g), gpu) if with_probs else None
+    parts = []
+    for c in counts:
+        parts += [torch.randint(0, m, (c,), generator=g, dtype=torch.int32),
+                  torch.zeros((c + 15) // 16 * 16 - c, dtype=torch.int32)]
+    idx = _dev(torch.cat(parts), gpu)
+    cnt = torch.tensor(counts, dtype=torch.int32, device=gpu)
+    plan = build_expert_plan(cnt, counts, pad=16)
+    a = permute(x, cnt, idx, counts, probs)
+    b = permute(x, cnt, idx, counts, probs, plan=plan)
+    torch.cuda.synchronize()
+    for u, v in zip(a, b):
+        assert (u is None) == (v is None)
+        if u is not None:
+            assert torch.equal(u.view(torch.uint8), v.view(torch.uint8))
+    with pytest.raises(ValueError):  # a plan of the other layout
+        permute(x, cnt, idx, counts, probs, plan=build_expert_plan(cnt, counts))
