@@ -7,6 +7,7 @@ gradient quantizer.
 import torch
 
 from ..utils.silu import (
+    build_expert_plan,
     triton_batch_weighted_silu_and_block_quant_backward,
     triton_batch_weighted_silu_and_block_quant_forward,
     triton_silu_and_block_quant_backward,
@@ -52,12 +53,16 @@ class BlockBatchWeightedSiluFunction(torch.autograd.Function):
     row.  Outputs keep the kernels' per-expert packing, so nothing is re-viewed.
     The quantizer lists are passed through to the tensor class; their first member
     gives the scale rounding and the FP8 format of all experts.  `plan` (optional, an
-    ExpertPlan of the same counts) is handed to the forward and kept for the backward."""
+    ExpertPlan of the same counts) is handed to the forward and kept for the backward; when
+    a backward will follow and the caller brought none, the forward builds one (one small
+    launch that both kernels gain more from than it costs)."""
 
     @staticmethod
     def forward(ctx, input, weights, counts, splits, quantizers, grad_quantizers, cls, is_recomputing, plan=None):
         lead = quantizers[0]
         ctx.save_for_backward(input, weights, counts)
+        if plan is None and (input.requires_grad or weights.requires_grad) and input.shape[0] > 0:
+            plan = build_expert_plan(counts, splits)
         ctx.sidecar = (splits, grad_quantizers, cls, input.requires_grad, plan)
         got = triton_batch_weighted_silu_and_block_quant_forward(
             input, weights, counts, splits=splits, round_scale=lead.force_pow_2_scales,
