@@ -230,7 +230,7 @@ def test_entry_points_under_graph_capture(gpu):
     between) must reproduce the eager results bit for bit."""
     from linghe_amd.quant.block import triton_blockwise_quant
     from linghe_amd.utils.norm import triton_rms_norm_and_block_quant_forward, triton_rms_norm_backward
-    from linghe_amd.utils.silu import (triton_batch_weighted_silu_and_block_quant_forward,
+    from linghe_amd.utils.silu import (build_expert_plan, triton_batch_weighted_silu_and_block_quant_forward,
                                        triton_silu_and_block_quant_backward)
 
     announce("graph capture and replay")
@@ -250,7 +250,10 @@ def test_entry_points_under_graph_capture(gpu):
         c = triton_batch_weighted_silu_and_block_quant_forward(inp, rw, cnt, counts)
         d = triton_rms_norm_backward(inp, inp, w)
         e = triton_blockwise_quant(inp)
-        return [t for grp in (a, b, c, d, e) for t in grp]
+        # the tile plan is one more launch on the stream, and the planned kernels only read it
+        plan = build_expert_plan(cnt, counts)
+        f = triton_batch_weighted_silu_and_block_quant_forward(inp, rw, cnt, counts, plan=plan)
+        return [t for grp in (a, b, c, d, e, f) for t in grp]
 
     def bits(ts):
         return [t.detach().clone().view(torch.uint8) if t.dtype != torch.float32 else t.detach().clone() for t in ts]
