@@ -236,7 +236,9 @@ def test_rmsnorm_fwd_bwd(gpu, M, N):
 
 
 @pytest.mark.parametrize("M,N", [(1024, 2048), (2048, 1536), (200, 512), (136, 7168), (128, 128), (256, 4096),
-                                 (64, 6144), (128, 8192), (72, 2176)])
+                                 (64, 6144), (128, 8192), (72, 2176),
+                                 # rows a multiple of 1024: both passes of mode 2 hand out the rows by XCD
+                                 (3072, 256), (5120, 640), (9216, 128)])
 @pytest.mark.parametrize("round_scale", [True, False])
 def test_rmsnorm_and_block_quant(gpu, M, N, round_scale):
     """reference tests/test_norm.py:189-220 (x = randn**2, weight randn, modes 0, 1, 2)."""
