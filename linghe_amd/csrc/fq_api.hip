@@ -59,7 +59,7 @@ int check_tiles(const char* fn, int64_t tiles) {
 
 extern "C" {
 
-int fq_version(void) { return 100; }
+int fq_version(void) { return 200; }  // 0.2.0: tile plans and the *_planned entry points
 
 const char* fq_last_error(void) { return g_err; }
 
