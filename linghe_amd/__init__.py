@@ -5,4 +5,4 @@ reference's wrappers (linghe.utils.norm, linghe.utils.silu, linghe.quant.block,
 linghe.quant.group) and call hand-written HIP kernels through the C ABI of
 libfq_gfx950.so (include/fq_api.h).
 """
-__version__ = "0.1.0"
+__version__ = "0.2.0"
